@@ -23,7 +23,8 @@ EXPORTS = (
     "misort_kernel_name",
     "misort_describe_plan",
     "misort_swap_last",
-    "misort_set_target_chunks",
+    "misort_scratch_bytes_chunked",
+    "misort_local_chunked",
     "misort_searchsorted",
     "misort_unique_scratch_bytes",
     "misort_unique",
@@ -114,8 +115,13 @@ def load():
     lib.misort_sort_axis.restype = c_int
     lib.misort_sort_axis.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t,
                                      c_int64, c_void_p]
-    lib.misort_set_target_chunks.restype = c_int
-    lib.misort_set_target_chunks.argtypes = [c_size_t]
+    lib.misort_scratch_bytes_chunked.restype = c_size_t
+    lib.misort_scratch_bytes_chunked.argtypes = [c_int, c_size_t, c_size_t, c_int, c_int, c_size_t]
+    lib.misort_local_chunked.restype = c_int
+    lib.misort_local_chunked.argtypes = [
+        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64,
+        c_void_p, c_size_t, c_void_p, c_size_t,
+    ]
     lib.misort_swap_last.restype = c_int
     lib.misort_swap_last.argtypes = [
         c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_size_t, c_size_t, c_void_p,

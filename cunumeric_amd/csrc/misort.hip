@@ -4,7 +4,6 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
-
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -218,8 +217,6 @@ struct Plan {
 #define MISORT_CHUNKS 512
 #endif
 static constexpr size_t kTargetChunks  = MISORT_CHUNKS;
-// chunks (workgroups) a radix pass over the whole array is cut into; misort_set_target_chunks
-static std::atomic<size_t> g_target_chunks{0};
 #ifndef MISORT_SLAB
 #define MISORT_SLAB 16
 #endif
@@ -232,8 +229,10 @@ static constexpr int kUpsweepThreads   = MISORT_UNT;
 static constexpr size_t kCount16MinLen = (size_t)1 << 20;
 static constexpr size_t kCount16Chunks = 512;
 
+// target_chunks: chunks (workgroups) a radix pass over the whole array is cut into; 0 = the
+// built-in choice.  It is part of the plan, so the scratch query and the sort must agree on it.
 static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsort,
-                     bool has_indices_in, Plan& pl)
+                     bool has_indices_in, Plan& pl, size_t target_chunks = 0)
 {
   if (!dtype_info(dtype, pl.dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
   pl.volume         = volume;
@@ -289,7 +288,7 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.n_passes      = pl.dt.bytes;  // 8-bit digits
     pl.tile          = tile_size(pl.dt.bytes, pl.pay);
     pl.tiles_per_row = (pl.row_len + pl.tile - 1) / pl.tile;
-    size_t target = g_target_chunks.load(std::memory_order_relaxed);
+    size_t target = target_chunks;
     if (target == 0) {
       // two workgroups per CU; one when that still leaves a workgroup fewer than four tiles
       // (measured: 2^24 int32 values 4 % faster, 2^26 and up 5 % slower with one)
@@ -382,42 +381,21 @@ constexpr bool is_float_width()
          std::is_same<KeyT, uint64_t>::value;
 }
 
-template <typename KeyT, int PAY>
-static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, const PassParams& pp)
+// the scatter kernel of one pass
+template <typename KeyT, int PAY, bool PART>
+static void launch_downsweep(Launcher& L, const Plan& pl, int id, bool first, bool last,
+                             const PassParams& pp)
 {
-  constexpr int NT   = TileCfg<sizeof(KeyT), PAY>::NT;
-  constexpr int IPT  = TileCfg<sizeof(KeyT), PAY>::IPT;
-  constexpr int OCC  = TileCfg<sizeof(KeyT), PAY>::OCC;
-  constexpr int G    = TileCfg<sizeof(KeyT), PAY>::G;
-  constexpr int TILE = NT * IPT;
-  constexpr int UNT  = kUpsweepThreads;
   const dim3 grid((unsigned)pl.n_chunks);
-  const dim3 sgrid((unsigned)(pl.rows * pl.slabs_per_row));
-
-  L.run(K_UPSWEEP, [&] {
-    if (first) {
-      if constexpr (is_float_width<KeyT>()) {
-        if (pl.specials) {
-          hipLaunchKernelGGL((upsweep_kernel<KeyT, true, true, UNT, TILE>), grid, dim3(UNT), 0,
-                             L.stream, pp);
-          return;
-        }
-      }
-      hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT, TILE>), grid, dim3(UNT), 0,
-                         L.stream, pp);
-    } else {
-      hipLaunchKernelGGL((upsweep_kernel<KeyT, false, false, UNT, TILE>), grid, dim3(UNT), 0,
-                         L.stream, pp);
-    }
-  });
-  L.run(K_SCAN_SLABS,
-        [&] { hipLaunchKernelGGL(chunk_scan_slabs, sgrid, dim3(RADIX), 0, L.stream, pp); });
-  L.run(K_SCAN_BASES,
-        [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
-
-  const int id = first ? (last ? K_DOWN_ONLY : K_DOWN_FIRST) : (last ? K_DOWN_LAST : K_DOWN_MIDDLE);
+  constexpr int NT  = TileCfg<sizeof(KeyT), PAY>::NT;
+  constexpr int IPT = TileCfg<sizeof(KeyT), PAY>::IPT;
+  constexpr int OCC = TileCfg<sizeof(KeyT), PAY>::OCC;
+  constexpr int G   = TileCfg<sizeof(KeyT), PAY>::G;
   L.run(id, [&] {
-    if (first && last)
+    if constexpr (PART)
+      hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, true, NT, IPT, G, OCC, true>), grid, dim3(NT),
+                         0, L.stream, pp);
+    else if (first && last)
       hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, true, NT, IPT, G, OCC>), grid, dim3(NT), 0,
                          L.stream, pp);
     else if (first)
@@ -430,6 +408,35 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
       hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, false, false, NT, IPT, G, OCC>), grid, dim3(NT),
                          0, L.stream, pp);
   });
+}
+
+template <typename KeyT, int PAY>
+static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, const PassParams& pp)
+{
+  constexpr int UNT = kUpsweepThreads;
+  const dim3 grid((unsigned)pl.n_chunks);
+  const dim3 sgrid((unsigned)(pl.rows * pl.slabs_per_row));
+
+  L.run(K_UPSWEEP, [&] {
+    if (first) {
+      if constexpr (is_float_width<KeyT>()) {
+        if (pl.specials) {
+          hipLaunchKernelGGL((upsweep_kernel<KeyT, true, true, UNT>), grid, dim3(UNT), 0, L.stream, pp);
+          return;
+        }
+      }
+      hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT>), grid, dim3(UNT), 0, L.stream, pp);
+    } else {
+      hipLaunchKernelGGL((upsweep_kernel<KeyT, false, false, UNT>), grid, dim3(UNT), 0, L.stream, pp);
+    }
+  });
+  L.run(K_SCAN_SLABS,
+        [&] { hipLaunchKernelGGL(chunk_scan_slabs, sgrid, dim3(RADIX), 0, L.stream, pp); });
+  L.run(K_SCAN_BASES,
+        [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
+
+  const int id = first ? (last ? K_DOWN_ONLY : K_DOWN_FIRST) : (last ? K_DOWN_LAST : K_DOWN_MIDDLE);
+  launch_downsweep<KeyT, PAY, false>(L, pl, id, first, last, pp);
 }
 
 static void launch_zero(Launcher& L, void* p, size_t bytes)
@@ -476,6 +483,7 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   pp.special_row     = special_row;
   pp.row_len         = pl.row_len;
   pp.index_offset    = a.index_offset;
+  pp.tile            = (uint32_t)pl.tile;
   pp.tiles_per_row   = (uint32_t)pl.tiles_per_row;
   pp.tiles_per_chunk = (uint32_t)pl.tiles_per_chunk;
   pp.chunks_per_row  = (uint32_t)pl.chunks_per_row;
@@ -543,15 +551,8 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
     cur_pay  = dst_pay;
   }
 
-  if (alias_keys)
-    L.run(K_COPY, [&] {
-      hipMemcpyAsync(vout, S + pl.off_keys[0], pl.volume * eb, hipMemcpyDeviceToDevice, L.stream);
-    });
-  if (alias_pay)
-    L.run(K_COPY, [&] {
-      hipMemcpyAsync(iout, S + pl.off_pay[0], pl.volume * pay_bytes, hipMemcpyDeviceToDevice,
-                     L.stream);
-    });
+  if (alias_keys) launch_copy(L, K_COPY, vout, S + pl.off_keys[0], pl.volume * eb);
+  if (alias_pay) launch_copy(L, K_COPY, iout, S + pl.off_pay[0], pl.volume * pay_bytes);
 
   if constexpr (is_float_width<KeyT>() && PAY == PAY_NONE) {
     if (pl.specials) {
@@ -725,11 +726,6 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
                                   void* pay_out, long long kth, int64_t index_offset, char* S)
 {
   const Plan& pl     = u.pl;
-  constexpr int NT   = TileCfg<sizeof(KeyT), PAY>::NT;
-  constexpr int IPT  = TileCfg<sizeof(KeyT), PAY>::IPT;
-  constexpr int OCC  = TileCfg<sizeof(KeyT), PAY>::OCC;
-  constexpr int G    = TileCfg<sizeof(KeyT), PAY>::G;
-  constexpr int TILE = NT * IPT;
   constexpr int UNT  = kUpsweepThreads;
   KeyT* pivot        = reinterpret_cast<KeyT*>(S + u.off_pivot);
   auto* kleft        = reinterpret_cast<unsigned long long*>(S + u.off_kleft);
@@ -765,6 +761,7 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
   pp.row_len         = pl.row_len;
   pp.index_offset    = index_offset;
+  pp.tile            = (uint32_t)pl.tile;
   pp.tiles_per_row   = (uint32_t)pl.tiles_per_row;
   pp.tiles_per_chunk = (uint32_t)pl.tiles_per_chunk;
   pp.chunks_per_row  = (uint32_t)pl.chunks_per_row;
@@ -775,17 +772,13 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.pivot           = pivot;
   const dim3 sgrid((unsigned)(pl.rows * pl.slabs_per_row));
   L.run(K_UPSWEEP, [&] {
-    hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT, TILE, true>), grid, dim3(UNT), 0, L.stream,
-                       pp);
+    hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT, true>), grid, dim3(UNT), 0, L.stream, pp);
   });
   L.run(K_SCAN_SLABS,
         [&] { hipLaunchKernelGGL(chunk_scan_slabs, sgrid, dim3(RADIX), 0, L.stream, pp); });
   L.run(K_SCAN_BASES,
         [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
-  L.run(K_SPLIT, [&] {
-    hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, true, NT, IPT, G, OCC, true>), grid, dim3(NT),
-                       0, L.stream, pp);
-  });
+  launch_downsweep<KeyT, PAY, true>(L, pl, K_SPLIT, true, true, pp);
 }
 
 template <typename KeyT>
@@ -803,11 +796,12 @@ static void partition_select_pay(Launcher& L, const PartLayout& u, const void* v
 // ---------------------------------------------------------------------------------------
 static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_out,
                     const int64_t* indices_in, int64_t* indices_out, size_t volume,
-                    size_t sort_dim_size, int64_t index_offset, void* scratch, size_t scratch_bytes)
+                    size_t sort_dim_size, int64_t index_offset, void* scratch, size_t scratch_bytes,
+                    size_t target_chunks = 0)
 {
   Plan pl;
   const bool argsort = indices_out != nullptr;
-  int rc = make_plan(dtype, volume, sort_dim_size, argsort, indices_in != nullptr, pl);
+  int rc = make_plan(dtype, volume, sort_dim_size, argsort, indices_in != nullptr, pl, target_chunks);
   if (rc != MISORT_OK) return rc;
   if (pl.strategy == S_EMPTY) return MISORT_OK;
 
@@ -871,10 +865,7 @@ static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_
         // complex keys-only: elements gathered by sorted position
         const void* src = values_in;
         if (values_in == values_out) {
-          L.run(K_COPY, [&] {
-            hipMemcpyAsync(a.scratch + pl.off_gather_src, values_in, volume * eb,
-                           hipMemcpyDeviceToDevice, L.stream);
-          });
+          launch_copy(L, K_COPY, a.scratch + pl.off_gather_src, values_in, volume * eb);
           src = a.scratch + pl.off_gather_src;
         }
         launch_gather(L, K_GATHER, eb, src, values_out,
@@ -925,6 +916,27 @@ int misort_local(int dtype, const void* values_in, void* values_out, const int64
   L.stream = reinterpret_cast<hipStream_t>(stream);
   return run_sort(L, dtype, values_in, values_out, indices_in, indices_out, volume, sort_dim_size,
                   index_offset, scratch, scratch_bytes);
+}
+
+size_t misort_scratch_bytes_chunked(int dtype, size_t volume, size_t sort_dim_size, int argsort,
+                                    int has_indices_in, size_t target_chunks)
+{
+  Plan pl;
+  if (make_plan(dtype, volume, sort_dim_size, argsort != 0, has_indices_in != 0, pl, target_chunks) !=
+      MISORT_OK)
+    return 0;
+  return pl.total;
+}
+
+int misort_local_chunked(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
+                         int64_t* indices_out, size_t volume, size_t sort_dim_size, int /*stable*/,
+                         int64_t index_offset, void* scratch, size_t scratch_bytes, void* stream,
+                         size_t target_chunks)
+{
+  Launcher L;
+  L.stream = reinterpret_cast<hipStream_t>(stream);
+  return run_sort(L, dtype, values_in, values_out, indices_in, indices_out, volume, sort_dim_size,
+                  index_offset, scratch, scratch_bytes, target_chunks);
 }
 
 int misort_local_profiled(int dtype, const void* values_in, void* values_out,
@@ -1044,10 +1056,15 @@ int misort_unique(int dtype, const void* values_in, void* values_out, unsigned l
   DtypeInfo dt;
   if (!dtype_info(dtype, dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
   if (!count_out) return fail(MISORT_ERR_NULL, "unique: count_out is NULL");
+  if (reinterpret_cast<uintptr_t>(count_out) % 8 != 0)
+    return fail(MISORT_ERR_ALIGN, "count_out not aligned to 8 bytes");
   Launcher L;
   L.stream = reinterpret_cast<hipStream_t>(stream);
   if (volume == 0) {
-    launch_zero(L, count_out, sizeof(unsigned long long));
+    // exactly the 8 bytes of the counter
+    L.run(K_ZERO, [&] {
+      hipLaunchKernelGGL(store_u64_kernel, dim3(1), dim3(1), 0, L.stream, count_out, 0ull);
+    });
     return L.err == hipSuccess ? MISORT_OK : fail(MISORT_ERR_RUNTIME, hipGetErrorString(L.err));
   }
   if (!values_in || !values_out || !scratch) return fail(MISORT_ERR_NULL, "unique: NULL pointer");
@@ -1056,8 +1073,6 @@ int misort_unique(int dtype, const void* values_in, void* values_out, unsigned l
   if (scratch_bytes < u.total) return fail(MISORT_ERR_SCRATCH, "unique: scratch too small");
   if (reinterpret_cast<uintptr_t>(scratch) % 256 != 0)
     return fail(MISORT_ERR_ALIGN, "scratch not aligned to 256 bytes");
-  if (reinterpret_cast<uintptr_t>(count_out) % 8 != 0)
-    return fail(MISORT_ERR_ALIGN, "count_out not aligned to 8 bytes");
   char* S      = reinterpret_cast<char*>(scratch);
   void* sorted = S + u.off_sorted;
   auto* blk    = reinterpret_cast<unsigned long long*>(S + u.off_blk);
@@ -1162,17 +1177,13 @@ int misort_partition(int dtype, const void* values_in, void* values_out, int64_t
   if (u.by_index) {
     const void* src = values_in;
     if (inplace) {
-      L.run(K_COPY, [&] {
-        hipMemcpyAsync(S + u.off_src, values_in, volume * eb, hipMemcpyDeviceToDevice, L.stream);
-      });
+      launch_copy(L, K_COPY, S + u.off_src, values_in, volume * eb);
       src = S + u.off_src;
     }
     launch_gather(L, K_GATHER, eb, src, values_out, reinterpret_cast<const int64_t*>(S + u.off_idx),
                   u.pl.rows, u.pl.row_len, 0);
   } else if (!want_indices && inplace) {
-    L.run(K_COPY, [&] {
-      hipMemcpyAsync(values_out, S + u.off_stage, volume * eb, hipMemcpyDeviceToDevice, L.stream);
-    });
+    launch_copy(L, K_COPY, values_out, S + u.off_stage, volume * eb);
   }
   if (L.err != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
@@ -1214,12 +1225,6 @@ int misort_sort_axis(int dtype, const void* values_in, void* values_out, int64_t
   return MISORT_OK;
 }
 
-int misort_set_target_chunks(size_t chunks)
-{
-  g_target_chunks.store(chunks, std::memory_order_relaxed);
-  return MISORT_OK;
-}
-
 int misort_swap_last(const void* in, void* out, size_t outer, size_t k, size_t mid, size_t l,
                      size_t elem_bytes, void* stream)
 {
@@ -1227,24 +1232,12 @@ int misort_swap_last(const void* in, void* out, size_t outer, size_t k, size_t m
   if (!in || !out) return fail(MISORT_ERR_NULL, "swap_last: NULL pointer");
   if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8 && elem_bytes != 16)
     return fail(MISORT_ERR_DTYPE, "swap_last: element size must be 1, 2, 4, 8 or 16");
-  if (k > 0x7FFFFFFFull || l > 0x7FFFFFFFull || mid > 0x7FFFFFFFull || outer * mid > 0x7FFFFFFFull ||
+  if (k > 0x7FFFFFFFull || l > 0x7FFFFFFFull || mid > 0x7FFFFFFFull ||
       ((k + 63) / 64) * ((l + 63) / 64) > 0x7FFFFFFFull)
     return fail(MISORT_ERR_UNSUPPORTED, "swap_last: extent too large");
   Launcher L;
   L.stream = reinterpret_cast<hipStream_t>(stream);
-  // grid.y carries outer * mid and is limited to 65535 per launch
-  const size_t plane = k * mid * l * elem_bytes;
-  const size_t per   = 65535 / mid;
-  if (per == 0) {
-    // mid alone exceeds one launch: one launch per (outer, chunk of mid) is not needed by the
-    // sort front-end (at most 4 dimensions), so this is reported instead of looped
-    return fail(MISORT_ERR_UNSUPPORTED, "swap_last: middle extent above 65535");
-  }
-  for (size_t o = 0; o < outer; o += per) {
-    const size_t n = outer - o < per ? outer - o : per;
-    launch_swap_last(L, K_TRANSPOSE, reinterpret_cast<const char*>(in) + o * plane,
-                     reinterpret_cast<char*>(out) + o * plane, n, k, mid, l, elem_bytes);
-  }
+  launch_swap_last(L, K_TRANSPOSE, in, out, outer, k, mid, l, elem_bytes);
   if (L.err != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
   return MISORT_OK;

@@ -56,6 +56,8 @@ __global__ void __launch_bounds__(256) zero_words_kernel(uint32_t* p, size_t n_w
     p4[i] = make_uint4(0, 0, 0, 0);
 }
 
+__global__ void store_u64_kernel(unsigned long long* p, unsigned long long v) { *p = v; }
+
 // ---------------------------------------------------------------------------------------
 // geometry shared by the three kernels of a pass
 // ---------------------------------------------------------------------------------------
@@ -71,6 +73,7 @@ struct PassParams {
   unsigned long long* special_row;  // [rows][4] {zeros, nans, negative zeros, negatives}
   uint64_t row_len;
   int64_t index_offset;
+  uint32_t tile;  // keys per tile of the downsweep
   uint32_t tiles_per_row;
   uint32_t tiles_per_chunk;
   uint32_t chunks_per_row;
@@ -124,7 +127,7 @@ __device__ __forceinline__ void lds_barrier()
 // and a private LDS histogram.  SPECIALS (first pass of a keys-only float sort) also counts
 // zeros / NaNs per wave sub-chunk for the patch that restores their bit patterns.
 // ---------------------------------------------------------------------------------------
-template <typename KeyT, bool FIRST, bool SPECIALS, int NT, int TILE, bool PART = false>
+template <typename KeyT, bool FIRST, bool SPECIALS, int NT, bool PART = false>
 __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
 {
   constexpr int NW = NT / 64;
@@ -140,7 +143,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   const uint32_t chunk = blockIdx.x % p.chunks_per_row;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const KeyT* in        = reinterpret_cast<const KeyT*>(p.keys_in) + (uint64_t)row * p.row_len;
-  const uint64_t clen   = (uint64_t)p.tiles_per_chunk * TILE;
+  const uint64_t clen   = (uint64_t)p.tiles_per_chunk * p.tile;
   // Counting zeros and NaNs needs each wavefront on a range of its own (their order is
   // rebuilt from per-wavefront counts); otherwise the wavefronts of the workgroup walk the
   // chunk together, one stream per workgroup.

@@ -65,6 +65,41 @@ static void launch_gather(Launcher& L, int id, size_t elem_bytes, const void* sr
 }
 
 // ---------------------------------------------------------------------------------------
+// plain device copy (staging buffers of the single-pass and in-place cases back to the
+// caller's array), in the widest unit both pointers and the size allow
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) copy_kernel(const T* __restrict__ src, T* __restrict__ dst, uint64_t n)
+{
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (uint64_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+static void launch_copy(Launcher& L, int id, void* dst, const void* src, size_t bytes)
+{
+  if (bytes == 0) return;
+  const uintptr_t mix = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes;
+  const size_t unit   = (mix & 15) == 0 ? 16 : (mix & 7) == 0 ? 8 : (mix & 3) == 0 ? 4 : (mix & 1) == 0 ? 2 : 1;
+  const uint64_t n    = bytes / unit;
+  size_t blocks       = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  L.run(id, [&] {
+#define MISORT_COPY_CASE(T)                                                                        \
+  hipLaunchKernelGGL(copy_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, L.stream, (const T*)src, \
+                     (T*)dst, n)
+    switch (unit) {
+      case 16: MISORT_COPY_CASE(u128); break;
+      case 8: MISORT_COPY_CASE(uint64_t); break;
+      case 4: MISORT_COPY_CASE(uint32_t); break;
+      case 2: MISORT_COPY_CASE(uint16_t); break;
+      default: MISORT_COPY_CASE(uint8_t); break;
+    }
+#undef MISORT_COPY_CASE
+  });
+}
+
+// ---------------------------------------------------------------------------------------
 // swap an axis with the last one: out[o][l][m][k] = in[o][k][m][l], 64 x 64 element tiles
 // of the (k, l) plane staged through LDS so that both the reads (along l) and the writes
 // (along k) are contiguous.  mid == 1 is a plain batched 2-D transpose.
@@ -74,28 +109,32 @@ static void launch_gather(Launcher& L, int id, size_t elem_bytes, const void* sr
 template <typename T>
 __global__ void __launch_bounds__(256)
 swap_last_kernel(const T* __restrict__ in, T* __restrict__ out, uint32_t K, uint32_t M, uint32_t L,
-                 uint32_t tiles_l)
+                 uint32_t tiles_l, uint64_t planes)
 {
   constexpr int TS = 64;
   __shared__ T tile[TS][TS + 1];
   const uint32_t tk = blockIdx.x / tiles_l, tl = blockIdx.x % tiles_l;
-  const uint32_t m = blockIdx.y % M, o = blockIdx.y / M;
-  const uint64_t plane = (uint64_t)K * M * L;
-  const T* src = in + (uint64_t)o * plane + (uint64_t)m * L;   // + k*M*L + l
-  T* dst       = out + (uint64_t)o * plane + (uint64_t)m * K;  // + l*M*K + k
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
-  const uint32_t l = tl * TS + tx;
-#pragma unroll 4
-  for (int j = ty; j < TS; j += 4) {
-    const uint32_t k = tk * TS + j;
-    if (k < K && l < L) tile[j][tx] = load_streaming(&src[(uint64_t)k * M * L + l]);
-  }
-  __syncthreads();
+  const uint32_t l  = tl * TS + tx;
   const uint32_t ko = tk * TS + tx;  // the fast index of the output
+  const uint64_t plane = (uint64_t)K * M * L;
+  // grid.y strides over the outer * mid planes (a launch dimension holds at most 65535)
+  for (uint64_t om = blockIdx.y; om < planes; om += gridDim.y) {
+    const uint64_t m = om % M, o = om / M;
+    const T* src = in + o * plane + m * L;   // + k*M*L + l
+    T* dst       = out + o * plane + m * K;  // + l*M*K + k
 #pragma unroll 4
-  for (int j = ty; j < TS; j += 4) {
-    const uint32_t lo = tl * TS + j;
-    if (lo < L && ko < K) dst[(uint64_t)lo * M * K + ko] = tile[tx][j];
+    for (int j = ty; j < TS; j += 4) {
+      const uint32_t k = tk * TS + j;
+      if (k < K && l < L) tile[j][tx] = load_streaming(&src[(uint64_t)k * M * L + l]);
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int j = ty; j < TS; j += 4) {
+      const uint32_t lo = tl * TS + j;
+      if (lo < L && ko < K) dst[(uint64_t)lo * M * K + ko] = tile[tx][j];
+    }
+    __syncthreads();
   }
 }
 
@@ -103,11 +142,12 @@ static void launch_swap_last(Launcher& L_, int id, const void* in, void* out, si
                              size_t M, size_t L, size_t elem_bytes)
 {
   const uint32_t tiles_k = (uint32_t)((K + 63) / 64), tiles_l = (uint32_t)((L + 63) / 64);
-  const dim3 grid(tiles_k * tiles_l, (unsigned)(outer * M));
+  const uint64_t planes  = (uint64_t)outer * M;
+  const dim3 grid(tiles_k * tiles_l, (unsigned)(planes < 65535 ? planes : 65535));
   L_.run(id, [&] {
 #define MISORT_SWAP_CASE(T)                                                                   \
   hipLaunchKernelGGL(swap_last_kernel<T>, grid, dim3(256), 0, L_.stream, (const T*)in, (T*)out, \
-                     (uint32_t)K, (uint32_t)M, (uint32_t)L, tiles_l)
+                     (uint32_t)K, (uint32_t)M, (uint32_t)L, tiles_l, planes)
     switch (elem_bytes) {
       case 1: MISORT_SWAP_CASE(uint8_t); break;
       case 2: MISORT_SWAP_CASE(uint16_t); break;

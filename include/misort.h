@@ -184,12 +184,21 @@ int misort_partition(int dtype, const void* values_in, void* values_out, int64_t
 int misort_sort_axis(int dtype, const void* values_in, void* values_out, int64_t* indices_out,
                      size_t outer, size_t k, size_t inner, int64_t index_offset, void* stream);
 
-/* Tuning knob, no counterpart in the reference: the number of chunks (one workgroup each)
- * that a radix pass over the whole array is cut into; a chunk is a run of consecutive
- * tiles that one workgroup walks in order.  0 restores the built-in choice.  Process-wide;
- * set it while no sort is being planned on another thread.  misort_scratch_bytes and
- * misort_local must see the same value. */
-int misort_set_target_chunks(size_t chunks);
+/*
+ * misort_scratch_bytes / misort_local with the number of chunks (one workgroup each) that a
+ * radix pass over the whole array is cut into given by the caller; a chunk is a run of
+ * consecutive tiles that one workgroup walks in order.  target_chunks == 0 is the built-in
+ * choice (two per CU), which is what the plain entry points use.  The value is part of the
+ * plan: give the same one to the query and to the sort.  No counterpart in the reference
+ * (CUB picks its grid itself, src/cunumeric/sort/cub_sort.cuh:60-71); for callers that
+ * share the GPU between several streams, and for tests of the multi-tile loop on small arrays.
+ */
+size_t misort_scratch_bytes_chunked(int dtype, size_t volume, size_t sort_dim_size, int argsort,
+                                    int has_indices_in, size_t target_chunks);
+int misort_local_chunked(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
+                         int64_t* indices_out, size_t volume, size_t sort_dim_size, int stable,
+                         int64_t index_offset, void* scratch, size_t scratch_bytes, void* stream,
+                         size_t target_chunks);
 
 /*
  * Dense row-major copy with one axis swapped with the last one:

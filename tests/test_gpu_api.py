@@ -301,3 +301,17 @@ class TestAllDtypes:
         a.flags.writeable = False
         with pytest.raises(ValueError):
             a.sort()
+
+
+# ---- shapes whose middle extent exceeds one launch dimension ---------------------------
+@pytest.mark.parametrize("dtype,shape", [(np.complex128, (2, 70000, 2)), (np.float64, (600, 70000, 2))],
+                         ids=["complex128", "float64"])
+def test_sort_axis0_with_a_long_middle_axis(dtype, shape):
+    """Sorting along axis 0 swaps it with the last axis; the planes of that copy (outer x
+    middle extent) exceed the 65535 blocks a launch dimension holds."""
+    rng = np.random.default_rng(91)
+    a = random_array(dtype, int(np.prod(shape)), rng).reshape(shape)
+    a_num = num.array(a)
+    assert bits_equal(np.asarray(num.sort(a_num, axis=0)), np.sort(a, axis=0, kind="stable"))
+    assert np.array_equal(np.asarray(num.argsort(a_num, axis=0, kind="stable")),
+                          np.argsort(a, axis=0, kind="stable"))

@@ -67,42 +67,39 @@ def test_rows(abi, dtype, rows, row_len):
     assert bits_equal(got, np.sort(a.reshape(rows, row_len), axis=1, kind="stable").reshape(-1))
 
 
-@pytest.fixture
-def few_chunks(abi):
-    """Cuts radix passes into 3 chunks, so that arrays of a few tiles already make every
-    workgroup walk several tiles (the pipelined loop, the carried partial lines and the
-    drain step) instead of the one tile per chunk that small arrays get by default."""
-    abi.lib.misort_set_target_chunks(3)
-    yield
-    abi.lib.misort_set_target_chunks(0)
+# Radix passes cut into 3 chunks (misort_local_chunked), so that arrays of a few tiles
+# already make every workgroup walk several tiles (the pipelined loop, the lines carried
+# from tile to tile and the final flush) instead of the one tile per chunk that small
+# arrays get by default.
+FEW = 3
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES, ids=lambda d: np.dtype(d).name)
-def test_multi_tile_chunks_all_dtypes(abi, few_chunks, dtype):
+def test_multi_tile_chunks_all_dtypes(abi, dtype):
     rng = np.random.default_rng(21)
     for n in (40000, 100003, 262144):
         print(f"multi-tile dtype={np.dtype(dtype).name} n={n}", flush=True)
         a = random_array(dtype, n, rng)
-        got = abi.local_sort(a, n, argsort=True)
+        got = abi.local_sort(a, n, argsort=True, chunks=FEW)
         assert np.array_equal(got, np.argsort(a, kind="stable")), (dtype, n)
-        got = abi.local_sort(a, n, argsort=False)
+        got = abi.local_sort(a, n, argsort=False, chunks=FEW)
         assert bits_equal(got, np.sort(a, kind="stable")), (dtype, n)
 
 
 @pytest.mark.parametrize("dtype", [np.uint8, np.float16, np.int32, np.float32, np.uint64, np.float64,
                                    np.complex64, np.complex128], ids=lambda d: np.dtype(d).name)
-def test_multi_tile_chunks_rows_and_payload(abi, few_chunks, dtype):
+def test_multi_tile_chunks_rows_and_payload(abi, dtype):
     rng = np.random.default_rng(22)
     rows, row_len = 3, 70001
     a = random_array(dtype, rows * row_len, rng).reshape(rows, row_len)
     print(f"multi-tile rows dtype={np.dtype(dtype).name}", flush=True)
-    got = abi.local_sort(a, row_len, argsort=False).reshape(rows, row_len)
+    got = abi.local_sort(a, row_len, argsort=False, chunks=FEW).reshape(rows, row_len)
     assert bits_equal(got, np.sort(a, axis=1, kind="stable"))
-    got = abi.local_sort(a, row_len, argsort=True).reshape(rows, row_len)
+    got = abi.local_sort(a, row_len, argsort=True, chunks=FEW).reshape(rows, row_len)
     assert np.array_equal(got, np.argsort(a, axis=1, kind="stable"))
     # caller-provided int64 payload travels with the keys
     pay = rng.integers(-(2**62), 2**62, rows * row_len, dtype=np.int64)
-    got = abi.local_sort(a, row_len, argsort=True, indices_in=pay).reshape(rows, row_len)
+    got = abi.local_sort(a, row_len, argsort=True, indices_in=pay, chunks=FEW).reshape(rows, row_len)
     ref = np.take_along_axis(pay.reshape(rows, row_len), np.argsort(a, axis=1, kind="stable"), axis=1)
     assert np.array_equal(got, ref)
 

@@ -89,3 +89,24 @@ def test_sizes_around_the_compaction_blocks(dtype):
             a = random_array(dtype, n, rng, narrow=narrow)
             print(f"unique dtype={np.dtype(dtype).name} n={n} narrow={narrow}", flush=True)
             assert same_values(num.unique(a), reference_unique(a)), (dtype, n, narrow)
+
+
+def test_abi_empty_input_writes_only_the_counter():
+    """misort_unique with volume 0 stores the 8-byte count and nothing beyond it."""
+    import torch
+
+    from cunumeric_amd import _lib
+    from cunumeric_amd.config import to_core_dtype
+
+    lib = _lib.load()
+    dev = torch.device("cuda", 0)
+    guard = torch.full((4,), 0x5A5A5A5A5A5A5A5A, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = lib.misort_unique(to_core_dtype(np.dtype(np.int32)), None, None, guard.data_ptr() + 8, 0, None, 0,
+                           stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert guard.cpu().tolist() == [0x5A5A5A5A5A5A5A5A, 0, 0x5A5A5A5A5A5A5A5A, 0x5A5A5A5A5A5A5A5A]
+    # a misaligned counter is refused before anything is written
+    assert lib.misort_unique(to_core_dtype(np.dtype(np.int32)), None, None, guard.data_ptr() + 4, 0, None,
+                             0, stream) == 5

@@ -79,7 +79,9 @@ class Abi:
         return t.from_numpy(a.reshape(-1).view(np.uint8).copy()).to(self.dev)
 
     def local_sort(self, values, sort_dim_size, argsort, indices_in=None, inplace=False,
-                   index_offset=0, want_values=False, profiled=False):
+                   index_offset=0, want_values=False, chunks=0, static=False):
+        """chunks != 0: misort_local_chunked with that chunk target; static: misort_local_static
+        (the library's own scratch)."""
         t = self.torch
         values = np.ascontiguousarray(values).reshape(-1)
         dt = values.dtype
@@ -98,13 +100,24 @@ class Abi:
                 d_iout = d_iin if inplace else t.empty(max(volume * 8, 16), dtype=t.uint8, device=self.dev)
             else:
                 d_iout = t.empty(max(volume * 8, 16), dtype=t.uint8, device=self.dev)
-        need = self.lib.misort_scratch_bytes(code, volume, sort_dim_size, int(argsort),
-                                             int(indices_in is not None))
-        scratch = t.empty(max(need, 256), dtype=t.uint8, device=self.dev)
         stream = t.cuda.current_stream().cuda_stream
         ptr = lambda x: None if x is None else x.data_ptr()
-        rc = self.lib.misort_local(code, ptr(d_in), ptr(d_vout), ptr(d_iin), ptr(d_iout), volume,
-                                   sort_dim_size, 1, index_offset, scratch.data_ptr(), need, stream)
+        if static:
+            rc = self.lib.misort_local_static(code, ptr(d_in), ptr(d_vout), ptr(d_iin), ptr(d_iout),
+                                              volume, sort_dim_size, 1, index_offset, stream)
+        elif chunks:
+            need = self.lib.misort_scratch_bytes_chunked(code, volume, sort_dim_size, int(argsort),
+                                                         int(indices_in is not None), chunks)
+            scratch = t.empty(max(need, 256), dtype=t.uint8, device=self.dev)
+            rc = self.lib.misort_local_chunked(code, ptr(d_in), ptr(d_vout), ptr(d_iin), ptr(d_iout),
+                                               volume, sort_dim_size, 1, index_offset,
+                                               scratch.data_ptr(), need, stream, chunks)
+        else:
+            need = self.lib.misort_scratch_bytes(code, volume, sort_dim_size, int(argsort),
+                                                 int(indices_in is not None))
+            scratch = t.empty(max(need, 256), dtype=t.uint8, device=self.dev)
+            rc = self.lib.misort_local(code, ptr(d_in), ptr(d_vout), ptr(d_iin), ptr(d_iout), volume,
+                                       sort_dim_size, 1, index_offset, scratch.data_ptr(), need, stream)
         self._lib.check(rc)
         t.cuda.synchronize()
         out_v = out_i = None
