@@ -25,6 +25,7 @@ EXPORTS = (
     "misort_swap_last",
     "misort_scratch_bytes_chunked",
     "misort_local_chunked",
+    "misort_local_static",
     "misort_searchsorted",
     "misort_unique_scratch_bytes",
     "misort_unique",
@@ -121,6 +122,10 @@ def load():
     lib.misort_local_chunked.argtypes = [
         c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64,
         c_void_p, c_size_t, c_void_p, c_size_t,
+    ]
+    lib.misort_local_static.restype = c_int
+    lib.misort_local_static.argtypes = [
+        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64, c_void_p,
     ]
     lib.misort_swap_last.restype = c_int
     lib.misort_swap_last.argtypes = [

@@ -885,6 +885,39 @@ static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_
 
 }  // namespace misort
 
+// ---------------------------------------------------------------------------------------
+// scratch that belongs to the library: misort_local_static sorts without any buffer from
+// the caller beyond the inputs and outputs, and without allocating.  One copy of the array
+// exists per GPU; in host code its name is only a handle for hipGetSymbolAddress.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char misort_static_scratch[MISORT_STATIC_SCRATCH_BYTES];
+
+namespace misort {
+
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_static_scratch_ptr[kMaxDevices];
+
+// Device address of misort_static_scratch on the current GPU, looked up once per GPU.
+static int static_scratch_address(void** out)
+{
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return fail(MISORT_ERR_RUNTIME, std::string("hipGetDevice: ") + hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(MISORT_ERR_UNSUPPORTED, "device ordinal above 63");
+  void* p = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(misort_static_scratch));
+    if (e != hipSuccess || !p)
+      return fail(MISORT_ERR_RUNTIME, std::string("hipGetSymbolAddress: ") + hipGetErrorString(e));
+    g_static_scratch_ptr[dev].store(p, std::memory_order_release);  // same value from any thread
+  }
+  *out = p;
+  return MISORT_OK;
+}
+
+}  // namespace misort
+
 using namespace misort;
 
 extern "C" {
@@ -916,6 +949,31 @@ int misort_local(int dtype, const void* values_in, void* values_out, const int64
   L.stream = reinterpret_cast<hipStream_t>(stream);
   return run_sort(L, dtype, values_in, values_out, indices_in, indices_out, volume, sort_dim_size,
                   index_offset, scratch, scratch_bytes);
+}
+
+int misort_local_static(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
+                        int64_t* indices_out, size_t volume, size_t sort_dim_size, int /*stable*/,
+                        int64_t index_offset, void* stream)
+{
+  Plan pl;
+  int rc = make_plan(dtype, volume, sort_dim_size, indices_out != nullptr, indices_in != nullptr, pl);
+  if (rc != MISORT_OK) return rc;
+  if (pl.total > (size_t)MISORT_STATIC_SCRATCH_BYTES) {
+    char msg[160];
+    snprintf(msg, sizeof msg,
+             "misort_local_static: this sort needs %zu bytes of scratch, the library's own buffer "
+             "holds %zu; use misort_local with a caller buffer",
+             pl.total, (size_t)MISORT_STATIC_SCRATCH_BYTES);
+    return fail(MISORT_ERR_SCRATCH, msg);
+  }
+  if (pl.strategy == S_EMPTY) return MISORT_OK;
+  void* own = nullptr;
+  rc        = static_scratch_address(&own);
+  if (rc != MISORT_OK) return rc;
+  Launcher L;
+  L.stream = reinterpret_cast<hipStream_t>(stream);
+  return run_sort(L, dtype, values_in, values_out, indices_in, indices_out, volume, sort_dim_size,
+                  index_offset, own, (size_t)MISORT_STATIC_SCRATCH_BYTES);
 }
 
 size_t misort_scratch_bytes_chunked(int dtype, size_t volume, size_t sort_dim_size, int argsort,

@@ -201,6 +201,24 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
                          size_t target_chunks);
 
 /*
+ * misort_local without a scratch argument and without any allocation: the scratch is a
+ * buffer of MISORT_STATIC_SCRATCH_BYTES that the library itself holds in device memory on
+ * every GPU it runs on, until the process ends.  No counterpart in the reference (which
+ * allocates from the Legate pool in every call, src/cunumeric/sort/cub_sort.cuh:46-62); it is
+ * for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same arguments and results as misort_local.  A sort
+ * whose misort_scratch_bytes exceeds MISORT_STATIC_SCRATCH_BYTES is refused with
+ * MISORT_ERR_SCRATCH (nothing is launched).  All calls on one GPU share the one buffer:
+ * calls that overlap in time on the same GPU (different streams or threads) race; calls
+ * ordered on one stream are safe.  The first call on a GPU looks the buffer's address up
+ * (hipGetSymbolAddress); no call uses hipMalloc, hipFree or an allocating library routine.
+ */
+#define MISORT_STATIC_SCRATCH_BYTES (64u << 20)
+int misort_local_static(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
+                        int64_t* indices_out, size_t volume, size_t sort_dim_size, int stable,
+                        int64_t index_offset, void* stream);
+
+/*
  * Dense row-major copy with one axis swapped with the last one:
  *   out[o][l][m][k] = in[o][k][m][l]   (in is outer x k x mid x l, out is outer x l x mid x k)
  * for elements of `elem_bytes` (1, 2, 4, 8 or 16) bytes.  mid == 1 is a batched 2-D
