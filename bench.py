@@ -6,8 +6,10 @@
 One "step" is one call of the hot path (misort_local through the C ABI) over the whole
 batch: float32 keys in HBM -> int64 stable-argsort indices in HBM.  Prints ONE JSON line.
 --workload selects one of the other benchmark inputs (c1, c3, c3t, c4, c5a, c5b) for the
-same line format; the default, c2, is the headline.  --calib-copy appends plain 1 GiB
-device copies, which give hardware-counter runs a kernel of known traffic to scale by.
+same line format; the default, c2, is the headline.  Every run of these workloads ends with
+plain 1 GiB device copies: their rate is reported beside the roofline, and they give
+hardware-counter runs a kernel of known traffic to scale by (--calib-copy is accepted for
+older command lines and changes nothing).
 
 Workload (the headline configuration): N = 2^28 float32, 98 % standard normal, 1 % NaN
 with random sign and payload bits, 0.5 % -0.0 and 0.5 % +0.0 at random positions, from a
@@ -93,10 +95,25 @@ def make_c5b(n: int = 1 << 30, seed: int = 6) -> np.ndarray:
 # ---------------------------------------------------------------------------------------
 # CPU baseline: the reference's CPU/OpenMP variant restated over Thrust's host back-ends
 # ---------------------------------------------------------------------------------------
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
+
+
 def cpu_baseline(sample: np.ndarray, code: int, row: int, argsort: bool, threads: int) -> dict:
+    """The reference's CPU/OpenMP variant (oracle/cpu_variant.cc: Thrust stable sort per row
+    under omp::par, as in sort_cpu.inl:40-69) timed on `threads` host cores: median of three
+    runs of std::chrono-equivalent wall time around the sort call only."""
     path = os.path.join(ROOT, "oracle", "libcpu_variant.so")
+    host = f"{cpu_model()}, {os.cpu_count()} logical CPUs on the host, {threads} threads used"
     if not os.path.exists(path):
-        return {"value": None, "unit": "Gkeys/s", "cores": threads, "kind": "port",
+        return {"value": None, "unit": "Gkeys/s", "cores": threads, "kind": "port", "host": host,
                 "sample": "oracle/libcpu_variant.so not built"}
     lib = ctypes.CDLL(path)
     lib.cpu_variant_sort.restype = ctypes.c_int
@@ -104,27 +121,40 @@ def cpu_baseline(sample: np.ndarray, code: int, row: int, argsort: bool, threads
                                      ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t,
                                      ctypes.c_int, ctypes.c_int]
     n = sample.size
+    note = ""
+    if sample.dtype.kind in "fc":
+        # Thrust's OpenMP merge sort compares with operator<, under which NaNs are unordered:
+        # its result on them is not a sort (and not what NumPy returns).  The baseline sorts the
+        # same input with every NaN replaced by a finite value, so that it times a real sort.
+        nan = np.isnan(sample)
+        if nan.any():
+            sample = sample.copy()
+            sample[nan] = 0.5
+            note = f"; its {int(nan.sum())} NaNs replaced by 0.5 (Thrust's omp merge sort does not order NaNs)"
     vals = np.empty_like(sample)
     idx = np.empty(n, dtype=np.int64) if argsort else None
-    best = None
-    for _ in range(2):
+    times = []
+    for _ in range(3):
         t0 = time.perf_counter()
         rc = lib.cpu_variant_sort(code, sample.ctypes.data, vals.ctypes.data,
                                   idx.ctypes.data if argsort else None, n, row, 1,
                                   1 if threads > 1 else 0)
         dt = time.perf_counter() - t0
         if rc != 0:
-            return {"value": None, "unit": "Gkeys/s", "cores": threads, "kind": "port",
+            return {"value": None, "unit": "Gkeys/s", "cores": threads, "kind": "port", "host": host,
                     "sample": "dtype not covered by the CPU variant port"}
-        best = dt if best is None else min(best, dt)
+        times.append(dt)
+    med = float(np.median(times))
     return {
-        "value": n / best / 1e9,
+        "value": n / med / 1e9,
         "unit": "Gkeys/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"first {n} elements of the same input (rows of {row}); thrust::stable_sort"
+        "host": host,
+        "sample": f"first {n} elements of the same input (rows of {row}){note}; thrust::stable_sort"
                   f"{'_by_key (int64 payload)' if argsort else ''} per row, omp::par, as in "
-                  f"sort_cpu.inl:40-69; {best*1e3:.0f} ms",
+                  f"sort_cpu.inl:40-69; median of 3 runs: {med*1e3:.0f} ms "
+                  f"({', '.join(f'{t*1e3:.0f}' for t in times)})",
     }
 
 
@@ -517,6 +547,22 @@ def main() -> int:
     ms_per_step = elapsed / args.steps * 1e3
     gkeys = n / (elapsed / args.steps) / 1e9
 
+    # One call at a time: HIP events on the launch stream (torch's current stream is the one
+    # handed to the library) from before the first launch to after the last kernel of the
+    # call, the device idle before each call; median over the calls.
+    n_ev = max(10, args.steps)
+    ev_ms = []
+    for _ in range(n_ev):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        step()
+        e1.record()
+        e1.synchronize()
+        ev_ms.append(e0.elapsed_time(e1))
+    call_ms = float(np.median(ev_ms))
+
     # quick parity guard on the timed output (the full oracle comparison lives in tests/):
     # argsort: the indices form a stable sorted order under the NumPy ordering;
     # sort: non-decreasing keys with the input's key checksum
@@ -560,7 +606,7 @@ def main() -> int:
         kms = (ctypes.c_float * max_k)()
         kid = (ctypes.c_int * max_k)()
         nk = ctypes.c_int(0)
-        reps = 5
+        reps = 10
         acc: dict = {}
         for _ in range(reps):
             _lib.check(lib.misort_local_profiled(code, d_in.data_ptr(), vo, None, io, n, row_len, 1, 0,
@@ -569,8 +615,15 @@ def main() -> int:
             for i in range(min(nk.value, max_k)):
                 name = lib.misort_kernel_name(kid[i]).decode()
                 acc.setdefault(name, []).append(kms[i])
-        kernels = {name: {"launches_per_step": len(v) // reps, "avg_ms": float(np.mean(v))}
-                   for name, v in acc.items()}
+        # avg_ms: median over the profiled calls of the mean duration of the kernel's launches
+        # in one call.  Every launch sits between two events here, and the device idles for
+        # the time an event takes between launches, so the sum over the kernels is an upper
+        # bound of the call (call_ms, timed without the inner events, is the figure to use).
+        kernels = {}
+        for name, v in acc.items():
+            per_call = np.asarray(v, dtype=np.float64).reshape(reps, -1)
+            kernels[name] = {"launches_per_step": per_call.shape[1],
+                             "avg_ms": float(np.median(per_call.mean(axis=1)))}
         all_ms = sum(k["avg_ms"] * k["launches_per_step"] for k in kernels.values())
 
         # roofline of the dominant kernel.  Radix plans: the downsweep scatter pass (all its
@@ -606,6 +659,8 @@ def main() -> int:
         b_total = tot_bytes / n + (k_bytes if n_up else 0)
         traffic = None
         if args.workload == "c2" and log2n == 28:
+            # from the rocprofv3 --pmc runs summarised in
+            # profiles/downsweep_c2_f32_argsort_2p28_hbm_traffic.md (not measurable from here)
             traffic = C2_DOWNSWEEP_TRAFFIC_BYTES_PER_LAUNCH
         elif args.workload == "c3" and log2n == 28:
             # measured: the row kernel reads 2 GiB and writes 2 GiB (FETCH_SIZE x2, WRITE_SIZE x1)
@@ -616,22 +671,38 @@ def main() -> int:
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
+            # frac prices a launch with the ALGORITHMIC bytes (int64 positions in every pass);
+            # frac_measured with the bytes the counters saw move (32-bit positions until the
+            # last pass): the second one is the achieved HBM bandwidth
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
+            "frac_measured": (traffic / (tot_ms / max(n_launch, 1) * 1e-3) / 1e9 / HBM_PEAK_GBS
+                              if traffic else None),
             "algorithmic_bytes_per_launch": tot_bytes / max(n_launch, 1),
             "avg_launch_ms": tot_ms / max(n_launch, 1),
             "per_pass": per_pass,
-            "whole_sort": {"bytes_per_key": b_total, "kernel_ms": all_ms,
-                           "GB/s": b_total * n / (all_ms * 1e-3) / 1e9 if all_ms else 0.0,
-                           "frac": b_total * n / (all_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if all_ms else 0.0},
+            # whole call: algorithmic bytes of all passes + one histogram read, over the time
+            # of one call from its first launch to its last kernel's end (HIP events)
+            "whole_sort": {"bytes_per_key": b_total, "call_ms": call_ms, "kernel_ms_sum": all_ms,
+                           "GB/s": b_total * n / (call_ms * 1e-3) / 1e9,
+                           "frac": b_total * n / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         }
 
-    if args.calib_copy:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
+    # what a plain device copy reaches on this box (1 GiB read + 1 GiB written per copy)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    c0 = torch.cuda.Event(enable_timing=True)
+    c1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    c0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    c1.record()
+    c1.synchronize()
+    copy_gbs = 10 * 2 * (1 << 30) / (c0.elapsed_time(c1) * 1e-3) / 1e9
+    del src, dst
 
     shape = f"N=2^{log2n}" if row == 0 else f"{n // 256} x 256"
     out = {
@@ -642,6 +713,11 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        # one call timed alone with HIP events (median of n), and its throughput
+        "call_ms_median": call_ms,
+        "call_ms_n": n_ev,
+        "value_per_call": n / (call_ms * 1e-3) / 1e9,
+        "device_copy_GBs": copy_gbs,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -26,6 +26,7 @@ EXPORTS = (
     "misort_scratch_bytes_chunked",
     "misort_local_chunked",
     "misort_local_static",
+    "misort_selftest_lds_lane_order",
     "misort_searchsorted",
     "misort_unique_scratch_bytes",
     "misort_unique",
@@ -127,6 +128,9 @@ def load():
     lib.misort_local_static.argtypes = [
         c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64, c_void_p,
     ]
+    lib.misort_selftest_lds_lane_order.restype = c_int
+    lib.misort_selftest_lds_lane_order.argtypes = [ctypes.c_uint, ctypes.POINTER(ctypes.c_ulonglong),
+                                                   ctypes.POINTER(ctypes.c_ulonglong), c_void_p]
     lib.misort_swap_last.restype = c_int
     lib.misort_swap_last.argtypes = [
         c_void_p, c_void_p, c_size_t, c_size_t, c_size_t, c_size_t, c_size_t, c_void_p,

@@ -5,6 +5,7 @@
 
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <type_traits>
@@ -20,12 +21,24 @@
 #include "search.hpp"
 #include "select.hpp"
 #include "unique.hpp"
+#include "selftest.hpp"
 
 namespace misort {
 
 static_assert(PAY_I64 == 2, "rows_api.hpp spells the caller-payload kind as 2");
 
 thread_local std::string g_last_error;
+
+// Ranking by returning LDS adds (radix.hpp, rank_by_add) is on unless the environment says
+// MISORT_RANK_BALLOT=1 when the library is first used; read once, never changed afterwards.
+static int rank_by_add_default()
+{
+  static const int v = [] {
+    const char* e = getenv("MISORT_RANK_BALLOT");
+    return (e && *e && *e != '0') ? 0 : 1;
+  }();
+  return v;
+}
 
 static int fail(int code, const std::string& msg)
 {
@@ -36,7 +49,6 @@ static int fail(int code, const std::string& msg)
 enum KernelId : int {
   K_ZERO = 0,
   K_UPSWEEP,
-  K_SCAN_SLABS,
   K_SCAN_BASES,
   K_DOWN_FIRST,
   K_DOWN_MIDDLE,
@@ -68,7 +80,7 @@ enum KernelId : int {
 };
 
 static const char* const kKernelNames[K_NUM] = {
-  "zero_words",      "upsweep",         "chunk_scan_slabs", "chunk_scan_bases",
+  "zero_words",      "upsweep",         "chunk_scan_bases",
   "downsweep_first", "downsweep_middle", "downsweep_last",  "downsweep_only",
   "rowsort_wave",    "rowsort_block",   "gather",           "copy",
   "swap_last",       "special_scan",    "special_collect",  "special_patch",
@@ -200,7 +212,8 @@ struct Plan {
   bool specials = false;  // float keys-only: patch original zero / NaN bit patterns back
   // scratch layout (byte offsets)
   size_t off_special_ctr = 0, special_ctr_bytes = 0;
-  size_t off_chunk_hist = 0, off_chunk_base = 0, off_slab_tot = 0;
+  size_t off_chunk_hist = 0, off_chunk_base = 0, off_slab_tot = 0, slab_tot_bytes = 0;
+  size_t zero_bytes = 0;  // from off_special_ctr on: what one launch clears before the first pass
   size_t off_keys[2] = {0, 0}, off_pay[2] = {0, 0};
   size_t off_special_blk = 0;
   size_t off_gather_idx = 0, off_gather_src = 0;
@@ -307,11 +320,15 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
         pl.tiles_per_row > 0xFFFFFFFFull)
       return fail(MISORT_ERR_UNSUPPORTED, "too many chunks for one launch");
 
+    // [special counters | slab totals of even passes | of odd passes]: cleared by one launch
     pl.special_ctr_bytes = pl.specials ? pl.rows * 4 * sizeof(unsigned long long) : 0;
     pl.off_special_ctr   = take(pl.special_ctr_bytes);
+    pl.slab_tot_bytes    = pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long);
+    pl.off_slab_tot      = take(pl.slab_tot_bytes);
+    take(pl.slab_tot_bytes);
+    pl.zero_bytes        = off - pl.off_special_ctr;
     pl.off_chunk_hist    = take(pl.n_chunks * RADIX * sizeof(uint32_t));
     pl.off_chunk_base    = take(pl.n_chunks * RADIX * sizeof(unsigned long long));
-    pl.off_slab_tot      = take(pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long));
 
     int n_bufs = pl.n_passes - 1 < 2 ? pl.n_passes - 1 : 2;
     if (n_bufs < 1) n_bufs = 1;  // single-pass sorts stage through one buffer when in == out
@@ -430,8 +447,6 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
       hipLaunchKernelGGL((upsweep_kernel<KeyT, false, false, UNT>), grid, dim3(UNT), 0, L.stream, pp);
     }
   });
-  L.run(K_SCAN_SLABS,
-        [&] { hipLaunchKernelGGL(chunk_scan_slabs, sgrid, dim3(RADIX), 0, L.stream, pp); });
   L.run(K_SCAN_BASES,
         [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
 
@@ -466,7 +481,7 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   unsigned long long* special_blk =
     reinterpret_cast<unsigned long long*>(S + pl.off_special_blk);
 
-  if (pl.specials) launch_zero(L, special_row, pl.special_ctr_bytes);
+  launch_zero(L, S + pl.off_special_ctr, pl.zero_bytes);
 
   const size_t pay_bytes     = PAY == PAY_IDX32 ? 4 : 8;
   const bool write_keys_last = !pl.argsort || a.values_out != nullptr;
@@ -478,7 +493,6 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   PassParams pp{};
   pp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
   pp.chunk_base      = reinterpret_cast<unsigned long long*>(S + pl.off_chunk_base);
-  pp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
   pp.special_blk     = pl.specials ? special_blk : nullptr;
   pp.special_row     = special_row;
   pp.row_len         = pl.row_len;
@@ -490,6 +504,7 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   pp.chunks_per_slab = (uint32_t)pl.chunks_per_slab;
   pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
   pp.xform           = pl.dt.xform;
+  pp.rank_by_add     = rank_by_add_default();
 
   const void* cur_keys = vin;
   const void* cur_pay  = iin;
@@ -522,6 +537,10 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
     pp.pay_in   = cur_pay;
     pp.pay_out  = dst_pay;
     pp.shift    = pass * RADIX_BITS;
+    pp.slab_tot = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + (pass & 1) * pl.slab_tot_bytes);
+    pp.slab_tot_next =
+      last ? nullptr
+           : reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + ((pass + 1) & 1) * pl.slab_tot_bytes);
     launch_pass<KeyT, PAY>(L, pl, first, last, pp);
 
     if constexpr (is_float_width<KeyT>() && PAY == PAY_NONE) {
@@ -711,9 +730,10 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   u.off_pivot       = take(pl.rows * 16);
   u.off_kleft       = take(pl.rows * sizeof(unsigned long long));
   u.off_ghist       = take(pl.rows * RADIX * sizeof(unsigned long long));
+  pl.slab_tot_bytes = pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long);
+  pl.off_slab_tot   = take(pl.slab_tot_bytes);  // cleared together with the counters before it
   pl.off_chunk_hist = take(pl.n_chunks * RADIX * sizeof(uint32_t));
   pl.off_chunk_base = take(pl.n_chunks * RADIX * sizeof(unsigned long long));
-  pl.off_slab_tot   = take(pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long));
   u.off_stage       = take(pl.volume * pl.dt.bytes);   // values when in == out
   u.off_idx         = take(pl.volume * sizeof(int64_t));  // positions when values are gathered
   u.off_src         = take(pl.volume * pl.dt.bytes);   // copy of the input for an in-place gather
@@ -734,7 +754,7 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   const dim3 rgrid((unsigned)pl.rows);
   const uint64_t clen = (uint64_t)pl.tiles_per_chunk * pl.tile;
 
-  launch_zero(L, ghist, pl.rows * RADIX * sizeof(unsigned long long));
+  launch_zero(L, ghist, pl.off_slab_tot + pl.slab_tot_bytes - u.off_ghist);
   L.run(K_SELECT_INIT, [&] {
     hipLaunchKernelGGL((select_init_kernel<KeyT>), dim3((unsigned)((pl.rows + 255) / 256)), dim3(256), 0,
                        L.stream, pivot, kleft, (uint32_t)pl.rows, (unsigned long long)kth);
@@ -759,6 +779,7 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
   pp.chunk_base      = reinterpret_cast<unsigned long long*>(S + pl.off_chunk_base);
   pp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
+  pp.slab_tot_next   = nullptr;
   pp.row_len         = pl.row_len;
   pp.index_offset    = index_offset;
   pp.tile            = (uint32_t)pl.tile;
@@ -774,8 +795,6 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   L.run(K_UPSWEEP, [&] {
     hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT, true>), grid, dim3(UNT), 0, L.stream, pp);
   });
-  L.run(K_SCAN_SLABS,
-        [&] { hipLaunchKernelGGL(chunk_scan_slabs, sgrid, dim3(RADIX), 0, L.stream, pp); });
   L.run(K_SCAN_BASES,
         [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
   launch_downsweep<KeyT, PAY, true>(L, pl, K_SPLIT, true, true, pp);
@@ -1280,6 +1299,30 @@ int misort_sort_axis(int dtype, const void* values_in, void* values_out, int64_t
   if (!served) return fail(MISORT_ERR_UNSUPPORTED, "sort_axis: axis too long for the column kernel");
   if (L.err != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
+  return MISORT_OK;
+}
+
+int misort_selftest_lds_lane_order(unsigned int rows_per_wave, unsigned long long* checked,
+                                   unsigned long long* out_of_order, void* stream)
+{
+  if (!checked || !out_of_order) return fail(MISORT_ERR_NULL, "selftest: NULL pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  unsigned long long* counts = nullptr;
+  hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&counts), HIP_SYMBOL(g_selftest_counts));
+  if (e != hipSuccess) return fail(MISORT_ERR_RUNTIME, std::string("hipGetSymbolAddress: ") + hipGetErrorString(e));
+  hipLaunchKernelGGL(store_u64_kernel, dim3(1), dim3(1), 0, st, counts, 0ull);
+  hipLaunchKernelGGL(store_u64_kernel, dim3(1), dim3(1), 0, st, counts + 1, 0ull);
+  // from all digit values distinct-ish down to every lane on one word
+  const uint32_t masks[6] = {0xFFu, 0x3Fu, 0x0Fu, 0x03u, 0x01u, 0x00u};
+  for (int i = 0; i < 6; ++i)
+    hipLaunchKernelGGL(lds_lane_order_probe_kernel, dim3(512), dim3(1024), 0, st, rows_per_wave, masks[i],
+                       0x1234567u + i, counts);
+  unsigned long long h[2] = {0, 0};
+  e = hipMemcpyAsync(h, counts, sizeof h, hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(e));
+  *checked      = h[0];
+  *out_of_order = h[1];
   return MISORT_OK;
 }
 

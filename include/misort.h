@@ -219,6 +219,20 @@ int misort_local_static(int dtype, const void* values_in, void* values_out, cons
                         int64_t index_offset, void* stream);
 
 /*
+ * Self test, no counterpart in the reference.  The radix scatter ranks the keys of a
+ * wavefront with one returning LDS add per key, which is stable only because gfx950 serves
+ * the lanes of one such instruction that hit the same word in ascending lane order.  This
+ * call checks exactly that on the current GPU: 6 x 512 workgroups x 16 wavefronts x
+ * rows_per_wave instructions with few distinct addresses, every lane compared with its rank
+ * by the ballot match.  *checked receives the number of lanes compared, *out_of_order the
+ * number that disagreed (0 on every MI355X seen).  Host pointers; synchronises `stream`.
+ * Setting MISORT_RANK_BALLOT=1 in the environment before the first call into the library
+ * makes every sort rank by ballots instead.
+ */
+int misort_selftest_lds_lane_order(unsigned int rows_per_wave, unsigned long long* checked,
+                                   unsigned long long* out_of_order, void* stream);
+
+/*
  * Dense row-major copy with one axis swapped with the last one:
  *   out[o][l][m][k] = in[o][k][m][l]   (in is outer x k x mid x l, out is outer x l x mid x k)
  * for elements of `elem_bytes` (1, 2, 4, 8 or 16) bytes.  mid == 1 is a batched 2-D
