@@ -50,6 +50,17 @@ def check_writeable(arr: "ndarray") -> None:
         raise ValueError("array is not writeable")
 
 
+def _reject_order(order, what: str) -> None:
+    """Structured-array field names have no meaning here (reference: cunumeric/deferred.py:3549-3553)."""
+    if order is not None:
+        raise NotImplementedError(f"{what}: 'order' is not supported, arrays hold plain numeric values")
+
+
+def _check_axis(axis, ndim: int) -> None:
+    if axis is not None and not -ndim <= axis < ndim:
+        raise ValueError(f"axis {axis} is out of bounds for an array of dimension {ndim}")
+
+
 class ndarray:
     """Dense C-ordered array in device memory (one HBM allocation, byte-addressed)."""
 
@@ -187,21 +198,12 @@ class ndarray:
         kind: str = "quicksort",
         order: Union[None, str, list] = None,
     ) -> None:
-        """(reference: cunumeric/deferred.py:3535-3557)"""
-        if kind == "stable":
-            stable = True
-        else:
-            stable = False
-
-        if order is not None:
-            raise NotImplementedError(
-                "cuNumeric does not support sorting with 'order' as "
-                "ndarray only supports numeric values"
-            )
-        if axis is not None and (axis >= rhs.ndim or axis < -rhs.ndim):
-            raise ValueError("invalid axis")
-
-        _sort_frontend(self, rhs, argsort, axis, stable)
+        """Same contract as the reference's thunk (cunumeric/deferred.py:3535-3557): only
+        the literal kind "stable" asks for stability, field names cannot be given (arrays
+        hold plain numbers), an axis outside the array is a ValueError."""
+        _reject_order(order, "sort")
+        _check_axis(axis, rhs.ndim)
+        _sort_frontend(self, rhs, argsort, axis, kind == "stable")
 
     def _thunk_partition(
         self,
@@ -215,13 +217,8 @@ class ndarray:
         """(reference: cunumeric/deferred.py:3559-3578, which does not look at ``kth`` and
         sorts.  Here a single in-range ``kth`` selects instead of sorting; a sequence of
         positions or an out-of-range one sorts, as the reference always does.)"""
-        if order is not None:
-            raise NotImplementedError(
-                "cuNumeric does not support partitioning with 'order' as "
-                "ndarray only supports numeric values"
-            )
-        if axis is not None and (axis >= rhs.ndim or axis < -rhs.ndim):
-            raise ValueError("invalid axis")
+        _reject_order(order, "partition")
+        _check_axis(axis, rhs.ndim)
 
         k: Optional[int] = None
         if isinstance(kth, (int, np.integer)) and not isinstance(kth, bool):
@@ -278,25 +275,24 @@ class ndarray:
         if side not in ("left", "right"):
             raise ValueError(f"side must be 'left' or 'right', not {side!r}")
         scalar = np.ndim(v) == 0 and not isinstance(v, (ndarray, torch.Tensor))
-        # this is needed in case v is a scalar
-        v_ndarray = convert_to_cunumeric_ndarray(v)
+        queries = convert_to_cunumeric_ndarray(v)  # a Python scalar becomes a 0-d array
         a = self
-        # in case we have different dtypes we need to find a common type
-        if a.dtype != v_ndarray.dtype:
-            ch_dtype = np.result_type(a.dtype, v_ndarray.dtype)
-            if v_ndarray.dtype != ch_dtype:
-                v_ndarray = v_ndarray.astype(ch_dtype)
-            if a.dtype != ch_dtype:
-                a = a.astype(ch_dtype)
+        # the kernel compares one element type: promote both sides to their common type
+        common = np.result_type(a.dtype, queries.dtype)
+        if queries.dtype != common:
+            queries = queries.astype(common)
+        if a.dtype != common:
+            a = a.astype(common)
         if sorter is not None and a.shape[0] > 1:
-            sorter = convert_to_cunumeric_ndarray(sorter)
-            if sorter.ndim != 1:
-                raise ValueError("Dimension mismatch: sorter must be a 1D array")
-            if sorter.shape != a.shape:
-                raise ValueError("Shape mismatch: sorter must have the same shape as self")
-            if not np.issubdtype(sorter.dtype, np.integer):
-                raise ValueError("Dtype mismatch: sorter must be of integer type")
-            a = a.take(sorter)
+            perm = convert_to_cunumeric_ndarray(sorter)
+            if perm.ndim != 1:
+                raise ValueError("sorter must be one-dimensional")
+            if perm.shape != a.shape:
+                raise ValueError("sorter must have as many elements as the array it sorts")
+            if not np.issubdtype(perm.dtype, np.integer):
+                raise ValueError("sorter must hold integers")
+            a = a.take(perm)
+        v_ndarray = queries
         result = ndarray(v_ndarray.shape, np.int64)
         if v_ndarray.size:
             _lib.check(

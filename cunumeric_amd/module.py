@@ -56,13 +56,11 @@ def sort_complex(a: Any) -> ndarray:
     promote to complex64, everything else to complex128
     (reference: cunumeric/module.py:7043-7078)."""
     result = sort(a)
-    # force complex result upon return
-    if np.issubdtype(result.dtype, np.complexfloating):
+    dt = result.dtype
+    if dt.kind == "c":
         return result
-    elif np.issubdtype(result.dtype, np.integer) and result.dtype.itemsize <= 2:
-        return result.astype(np.complex64, copy=True)
-    else:
-        return result.astype(np.complex128, copy=True)
+    narrow_int = dt.kind in "iu" and dt.itemsize <= 2
+    return result.astype(np.complex64 if narrow_int else np.complex128, copy=True)
 
 
 def argpartition(

@@ -152,7 +152,7 @@ def sort_task(output: "ndarray", input: "ndarray", argsort: bool, stable: bool,
     task.add_input(input)
     task.add_output(output)
     task.add_alignment(output, input)
-    task.add_scalar_arg(argsort)  # return indices flag
+    task.add_scalar_arg(argsort)
     task.add_scalar_arg(input.shape)
     task.add_scalar_arg(stable)
     task.execute()
@@ -169,14 +169,11 @@ def sort(
     """``kth`` (not in the reference, which sorts for partition): a position along the sort
     axis; when given, the rows are only partitioned around it."""
     if axis is None and input.ndim > 1:
+        # no axis: the array is sorted as one flat row
         sort_flattened(output, input, argsort, stable, kth)
-    else:
-        if axis is None:
-            computed_axis = 0
-        else:
-            computed_axis = normalize_axis_index(axis, input.ndim)
-
-        if computed_axis == input.ndim - 1:
-            sort_task(output, input, argsort, stable, kth)
-        elif not sort_along_axis(output, input, argsort, computed_axis):
-            sort_swapped(output, input, argsort, computed_axis, stable, kth)
+        return
+    ax = 0 if axis is None else normalize_axis_index(axis, input.ndim)
+    if ax == input.ndim - 1:
+        sort_task(output, input, argsort, stable, kth)       # rows are contiguous: sort them
+    elif not sort_along_axis(output, input, argsort, ax):     # short axis: sorted where it lies
+        sort_swapped(output, input, argsort, ax, stable, kth)  # else through a transposed copy
