@@ -1,0 +1,240 @@
+"""``quantile`` / ``percentile``: the callers of the sort path in the reference's statistics
+section (cunumeric/module.py:8339-8531 ``quantile``, 8534-8644 ``percentile``, which sort the
+array along the reduction axis with ``sort`` / ``ndarray.sort`` at :8472-8476 and then read
+the two order statistics around each quantile, ``quantile_impl`` :8248-8336).
+
+Same arguments, result shapes / dtypes and exceptions.  The order statistics come from the
+GPU sort of this package; for ONE quantile over a flat array or long rows they come from the
+selection behind ``partition`` instead (the reference's own comment at :8462-8467 names that
+as the cheaper way it does not take).  Picking the two neighbours out of the sorted array
+and blending them is elementwise arithmetic, which is not part of the sort path: it runs
+through torch on the device.  NumPy defines the 13 methods (numpy.quantile); the position of
+a quantile in the sorted sample and its blending weight follow NumPy's definitions, so
+results match numpy.quantile to rounding.
+"""
+from __future__ import annotations
+
+import math
+from typing import Any, Iterable, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from .array import _TORCH_TO_NUMPY, convert_to_cunumeric_ndarray, ndarray
+
+# Hyndman & Fan's plotting-position constants (alpha, beta) of the continuous methods: the
+# quantile q of n sorted samples sits at position n*q + alpha + q*(1 - alpha - beta) - 1.
+_CONTINUOUS = {
+    "interpolated_inverted_cdf": (0.0, 1.0),
+    "hazen": (0.5, 0.5),
+    "weibull": (0.0, 0.0),
+    "median_unbiased": (1.0 / 3.0, 1.0 / 3.0),
+    "normal_unbiased": (3.0 / 8.0, 3.0 / 8.0),
+}
+# methods that return one of the samples: the result keeps the input's dtype
+_SAMPLE_METHODS = ("inverted_cdf", "closest_observation", "lower", "higher", "nearest")
+METHODS = ("inverted_cdf", "averaged_inverted_cdf", "closest_observation", "interpolated_inverted_cdf",
+           "hazen", "weibull", "linear", "median_unbiased", "normal_unbiased", "lower", "higher",
+           "midpoint", "nearest")
+
+
+def _round_half_even(x: float) -> int:
+    f = math.floor(x)
+    d = x - f
+    if d > 0.5 or (d == 0.5 and f % 2 == 1):
+        return int(f) + 1
+    return int(f)
+
+
+def _position(method: str, q: float, n: int) -> tuple[int, int, float]:
+    """Where quantile ``q`` of ``n`` sorted samples lies: indices (lo, hi) of the two samples
+    and the weight g of the upper one; the quantile is lerp(x[lo], x[hi], g)."""
+    last = n - 1
+
+    def clipped(v: float, weight) -> tuple[int, int, float]:
+        # beyond the ends the quantile is the extreme sample
+        if v >= last:
+            return last, last, 0.0
+        if v < 0:
+            return 0, 0, 0.0
+        lo = math.floor(v)
+        return int(lo), int(lo) + 1, weight(v - lo, v)
+
+    if method in _CONTINUOUS or method == "linear":
+        if method == "linear":
+            v = last * q  # same position as alpha = beta = 1, with less rounding
+        else:
+            alpha, beta = _CONTINUOUS[method]
+            v = n * q + (alpha + q * (1.0 - alpha - beta)) - 1.0
+        return clipped(v, lambda frac, _: frac)
+    if method == "averaged_inverted_cdf":
+        return clipped(n * q - 1.0, lambda frac, _: 0.5 if frac == 0 else 1.0)
+    if method == "midpoint":
+        v = 0.5 * (math.floor(last * q) + math.ceil(last * q))
+        return clipped(v, lambda frac, vv: 0.0 if vv % 1 == 0 else 0.5)
+    # the remaining methods name one sample
+    if method == "inverted_cdf":
+        v = n * q - 1.0
+        lo = math.floor(v)
+        i = lo if v == lo else lo + 1
+    elif method == "closest_observation":
+        v = n * q - 1.5
+        lo = math.floor(v)
+        # on a tie take the order statistic with the even 1-based rank
+        i = lo if (v == lo and lo % 2 == 1) else lo + 1
+    elif method == "lower":
+        i = math.floor(last * q)
+    elif method == "higher":
+        i = math.ceil(last * q)
+    elif method == "nearest":
+        i = _round_half_even(last * q)
+    else:
+        raise ValueError(f"{method!r} is not a valid method. Use one of: {', '.join(METHODS)}")
+    i = min(max(int(i), 0), last)
+    return i, i, 0.0
+
+
+def _torch_dtype(dtype) -> torch.dtype:
+    for t, n in _TORCH_TO_NUMPY.items():
+        if np.dtype(n) == np.dtype(dtype):
+            return t
+    raise TypeError(dtype)
+
+
+def _from_torch(t: torch.Tensor, dtype) -> ndarray:
+    t = t.contiguous()
+    return ndarray(tuple(t.shape), dtype, _buf=t.reshape(-1).view(torch.uint8))
+
+
+def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool) -> dict[int, torch.Tensor]:
+    """``a`` has the reduction axis last: the samples at the sorted positions ``wanted`` of
+    every row, as tensors of the row shape.  One or two adjacent positions on long rows are
+    found by selection (partition around the lower one; the upper one is then the smallest
+    element behind it); anything else sorts the rows."""
+    from .module import partition, sort
+
+    n = a.shape[-1]
+    wanted = sorted(set(wanted))
+    # (signed integers and floats: the reduction that picks the upper neighbour is a torch op)
+    select = (len(wanted) <= 2 and wanted[-1] - wanted[0] <= 1 and n >= (1 << 16) and
+              a.dtype.itemsize >= 4 and a.dtype.kind in "fi")
+    if select:
+        k = wanted[0]
+        if overwrite_input:
+            a.partition(k, axis=-1)
+            part = a
+        else:
+            part = partition(a, k, axis=-1)
+        t = part.to_torch()
+        out = {k: t[..., k]}
+        if len(wanted) == 2:
+            out[k + 1] = t[..., k + 1:].amin(dim=-1)
+        return out
+    if overwrite_input:
+        a.sort(axis=-1)
+        s = a
+    else:
+        s = sort(a, axis=-1)
+    t = s.to_torch()
+    return {k: t[..., k] for k in wanted}
+
+
+def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: Optional[ndarray] = None,
+             overwrite_input: bool = False, method: str = "linear", keepdims: bool = False) -> ndarray:
+    """The q-th quantile(s) of ``a`` along ``axis`` (``None``: of the flattened array; several
+    axes: of their product).  Result shape: ``q.shape`` followed by the shape of ``a`` without
+    the reduced axes (kept with extent 1 under ``keepdims``); dtype: the input's for the methods
+    that return a sample, float64 otherwise; complex input is a TypeError, a wrongly shaped
+    ``out`` a ValueError (reference: cunumeric/module.py:8339-8531)."""
+    if method not in METHODS:
+        raise ValueError(f"{method!r} is not a valid method. Use one of: {', '.join(METHODS)}")
+    a = convert_to_cunumeric_ndarray(a)
+    if a.dtype.kind == "c":
+        raise TypeError("input array cannot be of complex type")
+    q_arr = np.asarray(q, dtype=np.float64)
+    if q_arr.size and not (np.all(q_arr >= 0) and np.all(q_arr <= 1)):
+        raise ValueError("Quantiles must be in the range [0, 1]")
+    original_shape = a.shape
+    nd = a.ndim
+
+    # ---- the reduction axes last, merged into one --------------------------------------
+    if axis is None:
+        axes = tuple(range(nd))
+    elif isinstance(axis, Iterable):
+        axes = tuple(int(x) for x in axis)
+    else:
+        axes = (int(axis),)
+    norm = []
+    for x in axes:
+        if not -nd <= x < nd:
+            raise ValueError(f"axis {x} is out of bounds for an array of dimension {nd}")
+        norm.append(x % nd if nd else 0)
+    if len(set(norm)) != len(norm):
+        raise ValueError("repeated axis")
+    axes = tuple(norm)
+    kept = tuple(k for k in range(nd) if k not in axes)
+    n = 1
+    for k in axes:
+        n *= original_shape[k]
+    if nd == 0:
+        n = 1
+    if n == 0:
+        raise ValueError("cannot take a quantile of an empty sample")
+    kept_shape = tuple(original_shape[k] for k in kept)
+    if nd and (kept + axes) != tuple(range(nd)):
+        # a dense copy with the reduced axes moved behind the others (never sorted in place)
+        moved = a.to_torch().permute(*kept, *axes).contiguous()
+        rows = _from_torch(moved.reshape(*kept_shape, n), a.dtype)
+        overwrite_input = False
+    else:
+        rows = a.reshape((*kept_shape, n))
+        if len(axes) > 1 and axis is not None:
+            overwrite_input = False  # as the reference: only a single axis is sorted in place
+
+    # ---- the samples around every quantile ---------------------------------------------
+    places = [_position(method, float(qv), n) for qv in q_arr.reshape(-1)]
+    wanted = [p[0] for p in places] + [p[1] for p in places]
+    stats = _order_statistics(rows, wanted, overwrite_input)
+    to_dtype = a.dtype if method in _SAMPLE_METHODS else np.dtype(np.float64)
+    tdt = _torch_dtype(to_dtype)
+    results = []
+    for lo, hi, g in places:
+        if lo == hi or g == 0.0:
+            r = stats[lo].to(tdt)
+        else:
+            x, y = stats[lo].to(tdt), stats[hi].to(tdt)
+            d = y - x
+            # the upper sample anchors the blend from the middle on, as in NumPy
+            r = x + d * g if g < 0.5 else y - d * (1.0 - g)
+        results.append(r)
+    res = torch.stack(results, dim=0) if results else torch.empty((0, *kept_shape), dtype=tdt,
+                                                                  device=rows.to_torch().device)
+    if a.dtype.kind == "f":
+        # a sample with a NaN has no quantiles: its largest element (NaNs sort last) tells
+        has_nan = torch.isnan(rows.to_torch()).any(dim=-1) if rows.size else None
+        if has_nan is not None and bool(has_nan.any()):
+            nan = torch.tensor(float("nan"), dtype=tdt, device=res.device)
+            res = torch.where(has_nan.unsqueeze(0), nan, res)
+    if keepdims:
+        remaining = tuple(1 if k in axes else original_shape[k] for k in range(nd))
+    else:
+        remaining = kept_shape
+    shape = (*q_arr.shape, *remaining)
+    res = res.reshape(shape)
+    if out is not None:
+        if tuple(out.shape) != shape:
+            raise ValueError("wrong shape on output array")
+        out.to_torch().copy_(res.to(_torch_dtype(out.dtype)))
+        return out
+    return _from_torch(res, to_dtype)
+
+
+def percentile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: Optional[ndarray] = None,
+               overwrite_input: bool = False, method: str = "linear", keepdims: bool = False) -> ndarray:
+    """The q-th percentile(s): ``quantile`` with ``q / 100``
+    (reference: cunumeric/module.py:8534-8644)."""
+    q_arr = np.true_divide(np.asarray(q, dtype=np.float64), 100.0)
+    if q_arr.size and not (np.all(q_arr >= 0) and np.all(q_arr <= 1)):
+        raise ValueError("Percentiles must be in the range [0, 100]")
+    return quantile(a, q_arr, axis=axis, out=out, overwrite_input=overwrite_input, method=method,
+                    keepdims=keepdims)
