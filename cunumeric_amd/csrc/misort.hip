@@ -49,7 +49,6 @@ static int fail(int code, const std::string& msg)
 enum KernelId : int {
   K_ZERO = 0,
   K_UPSWEEP,
-  K_SCAN_BASES,
   K_DOWN_FIRST,
   K_DOWN_MIDDLE,
   K_DOWN_LAST,
@@ -80,7 +79,7 @@ enum KernelId : int {
 };
 
 static const char* const kKernelNames[K_NUM] = {
-  "zero_words",      "upsweep",         "chunk_scan_bases",
+  "zero_words",      "upsweep",
   "downsweep_first", "downsweep_middle", "downsweep_last",  "downsweep_only",
   "rowsort_wave",    "rowsort_block",   "gather",           "copy",
   "swap_last",       "special_scan",    "special_collect",  "special_patch",
@@ -212,7 +211,7 @@ struct Plan {
   bool specials = false;  // float keys-only: patch original zero / NaN bit patterns back
   // scratch layout (byte offsets)
   size_t off_special_ctr = 0, special_ctr_bytes = 0;
-  size_t off_chunk_hist = 0, off_chunk_base = 0, off_slab_tot = 0, slab_tot_bytes = 0;
+  size_t off_chunk_hist = 0, off_slab_tot = 0, slab_tot_bytes = 0;
   size_t zero_bytes = 0;  // from off_special_ctr on: what one launch clears before the first pass
   size_t off_keys[2] = {0, 0}, off_pay[2] = {0, 0};
   size_t off_special_blk = 0;
@@ -328,7 +327,6 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     take(pl.slab_tot_bytes);
     pl.zero_bytes        = off - pl.off_special_ctr;
     pl.off_chunk_hist    = take(pl.n_chunks * RADIX * sizeof(uint32_t));
-    pl.off_chunk_base    = take(pl.n_chunks * RADIX * sizeof(unsigned long long));
 
     int n_bufs = pl.n_passes - 1 < 2 ? pl.n_passes - 1 : 2;
     if (n_bufs < 1) n_bufs = 1;  // single-pass sorts stage through one buffer when in == out
@@ -432,7 +430,6 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
 {
   constexpr int UNT = kUpsweepThreads;
   const dim3 grid((unsigned)pl.n_chunks);
-  const dim3 sgrid((unsigned)(pl.rows * pl.slabs_per_row));
 
   L.run(K_UPSWEEP, [&] {
     if (first) {
@@ -447,8 +444,6 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
       hipLaunchKernelGGL((upsweep_kernel<KeyT, false, false, UNT>), grid, dim3(UNT), 0, L.stream, pp);
     }
   });
-  L.run(K_SCAN_BASES,
-        [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
 
   const int id = first ? (last ? K_DOWN_ONLY : K_DOWN_FIRST) : (last ? K_DOWN_LAST : K_DOWN_MIDDLE);
   launch_downsweep<KeyT, PAY, false>(L, pl, id, first, last, pp);
@@ -492,7 +487,6 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
 
   PassParams pp{};
   pp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
-  pp.chunk_base      = reinterpret_cast<unsigned long long*>(S + pl.off_chunk_base);
   pp.special_blk     = pl.specials ? special_blk : nullptr;
   pp.special_row     = special_row;
   pp.row_len         = pl.row_len;
@@ -733,7 +727,6 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   pl.slab_tot_bytes = pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long);
   pl.off_slab_tot   = take(pl.slab_tot_bytes);  // cleared together with the counters before it
   pl.off_chunk_hist = take(pl.n_chunks * RADIX * sizeof(uint32_t));
-  pl.off_chunk_base = take(pl.n_chunks * RADIX * sizeof(unsigned long long));
   u.off_stage       = take(pl.volume * pl.dt.bytes);   // values when in == out
   u.off_idx         = take(pl.volume * sizeof(int64_t));  // positions when values are gathered
   u.off_src         = take(pl.volume * pl.dt.bytes);   // copy of the input for an in-place gather
@@ -777,7 +770,6 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.pay_in          = nullptr;
   pp.pay_out         = pay_out;
   pp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
-  pp.chunk_base      = reinterpret_cast<unsigned long long*>(S + pl.off_chunk_base);
   pp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
   pp.slab_tot_next   = nullptr;
   pp.row_len         = pl.row_len;
@@ -791,12 +783,9 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.xform           = pl.dt.xform;
   pp.shift           = 0;
   pp.pivot           = pivot;
-  const dim3 sgrid((unsigned)(pl.rows * pl.slabs_per_row));
   L.run(K_UPSWEEP, [&] {
     hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT, true>), grid, dim3(UNT), 0, L.stream, pp);
   });
-  L.run(K_SCAN_BASES,
-        [&] { hipLaunchKernelGGL(chunk_scan_bases, sgrid, dim3(RADIX), 0, L.stream, pp); });
   launch_downsweep<KeyT, PAY, true>(L, pl, K_SPLIT, true, true, pp);
 }
 
