@@ -176,7 +176,7 @@ WORKLOADS = {
 # HBM bytes per launch of the downsweep kernel on the headline workload (N = 2^28), from
 # the FETCH_SIZE / WRITE_SIZE hardware counters scaled by what the same counters read for
 # a 1 GiB copy; profiles/downsweep_c2_f32_argsort_2p28_hbm_traffic.md holds the runs.
-C2_DOWNSWEEP_TRAFFIC_BYTES_PER_LAUNCH = 4.145e9  # 1.751 GiB read + 2.110 GiB written
+C2_DOWNSWEEP_TRAFFIC_BYTES_PER_LAUNCH = 4.153e9  # 1.752 GiB read + 2.116 GiB written
 
 
 def algorithmic_bytes_per_key(k: int, v: int, role: str) -> int:
