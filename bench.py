@@ -465,6 +465,27 @@ def run_axis(args) -> int:
     return 0 if ok else 1
 
 
+def gpu_library_baseline(workload: str, log2n: int):
+    """The reference's device work for this workload (index fill + copy + CUB radix sort,
+    src/cunumeric/sort/sort.cu:1694-1751 and cub_sort.cuh:36-189) served by hipCUB / rocPRIM on
+    this GPU: oracle/hipcub_calls, a separate program run as a child process after the timed
+    region.  A reported comparison, like cpu_baseline; None when the program is not built or
+    has no case for the workload."""
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "hipcub_calls")
+    if workload not in ("c1", "c2", "c4") or not os.access(exe, os.X_OK):
+        return None
+    import subprocess
+    try:
+        r = subprocess.run([exe, workload, str(log2n), "10"], capture_output=True, text=True, timeout=300)
+        d = json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as e:  # a baseline that does not run is reported, not fatal
+        return {"value": None, "unit": "Gkeys/s", "kind": "hipcub", "error": str(e)[:200]}
+    return {"value": d["Gkeys_per_s"], "unit": "Gkeys/s", "kind": "hipcub (rocPRIM) DeviceRadixSort, the "
+            "reference's call sequence", "ms_median": d["ms_median"], "library_call_only_ms":
+            d["library_call_only_ms"], "calls": d["calls"], "sample": f"2^{log2n} keys of the same "
+            "distribution, generated on the device"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -739,6 +760,9 @@ def main() -> int:
                                    "sample": "see --workload c3"}
         else:
             out["cpu_baseline"] = cpu_baseline(flat[:sample_n], code, cpu_row, argsort, threads)
+        lib_base = gpu_library_baseline(args.workload, log2n)
+        if lib_base is not None:
+            out["gpu_library_baseline"] = lib_base
     print(json.dumps(out))
     return 0 if ok else 1
 
