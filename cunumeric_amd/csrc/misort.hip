@@ -40,6 +40,17 @@ static int rank_by_add_default()
   return v;
 }
 
+// The digit side-band of keys-only sorts (radix.hpp, SIDE) is on unless the environment says
+// MISORT_SIDE_BAND=0 when the library is first used.
+static bool side_band_default()
+{
+  static const bool v = [] {
+    const char* e = getenv("MISORT_SIDE_BAND");
+    return !(e && *e == '0');
+  }();
+  return v;
+}
+
 static int fail(int code, const std::string& msg)
 {
   g_last_error = msg;
@@ -215,6 +226,10 @@ struct Plan {
   size_t zero_bytes = 0;  // from off_special_ctr on: what one launch clears before the first pass
   size_t off_keys[2] = {0, 0}, off_pay[2] = {0, 0};
   size_t off_special_blk = 0;
+  // digit side-band of keys-only sorts: one byte per key, written by every pass but the last
+  // and counted by the next pass's upsweep in place of the keys
+  bool side_band = false;
+  size_t off_digits = 0;
   size_t off_gather_idx = 0, off_gather_src = 0;
   // counting sort of 2-byte keys: chunks of the histogram kernel, counters, their scan
   size_t c16_chunks = 0, c16_chunk_len = 0, off_c16_hist = 0, off_c16_prefix = 0;
@@ -237,6 +252,10 @@ static constexpr size_t kChunksPerSlab = MISORT_SLAB;
 #define MISORT_UNT 256
 #endif
 static constexpr int kUpsweepThreads   = MISORT_UNT;
+#ifndef MISORT_UDT
+#define MISORT_UDT 256
+#endif
+static constexpr int kUpsweepDigitThreads = MISORT_UDT;  // upsweep over the digit side-band
 // values-only sorts of 2-byte elements: counted instead of radix-sorted from this length on
 static constexpr size_t kCount16MinLen = (size_t)1 << 20;
 static constexpr size_t kCount16Chunks = 512;
@@ -340,6 +359,10 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
       for (int b = 0; b < n_pbufs; ++b) pl.off_pay[b] = take(pl.volume * pb);
       if (n_pbufs == 1) pl.off_pay[1] = pl.off_pay[0];
     }
+    // (8-byte keys: the upsweep saves 7 of 8 bytes per key; with 4-byte keys the extra
+    // stores of the scatter cost more than the upsweep saves)
+    pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
+    if (pl.side_band) pl.off_digits = take(pl.volume);
     if (pl.specials)
       pl.off_special_blk =
         take(pl.n_chunks * (kUpsweepThreads / 64) * 2 * sizeof(unsigned long long));
@@ -407,6 +430,17 @@ static void launch_downsweep(Launcher& L, const Plan& pl, int id, bool first, bo
   constexpr int OCC = TileCfg<sizeof(KeyT), PAY>::OCC;
   constexpr int G   = TileCfg<sizeof(KeyT), PAY>::G;
   L.run(id, [&] {
+    if constexpr (!PART && PAY == PAY_NONE && sizeof(KeyT) == 8) {
+      if (pp.digits_out) {  // keys-only pass that also writes the digit side-band
+        if (first)
+          hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, false, NT, IPT, G, OCC, false, true>), grid,
+                             dim3(NT), 0, L.stream, pp);
+        else
+          hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, false, false, NT, IPT, G, OCC, false, true>), grid,
+                             dim3(NT), 0, L.stream, pp);
+        return;
+      }
+    }
     if constexpr (PART)
       hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, true, NT, IPT, G, OCC, true>), grid, dim3(NT),
                          0, L.stream, pp);
@@ -432,6 +466,11 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
   const dim3 grid((unsigned)pl.n_chunks);
 
   L.run(K_UPSWEEP, [&] {
+    if (pp.digits_in) {
+      hipLaunchKernelGGL((upsweep_digits_kernel<kUpsweepDigitThreads>), grid, dim3(kUpsweepDigitThreads), 0,
+                         L.stream, pp);
+      return;
+    }
     if (first) {
       if constexpr (is_float_width<KeyT>()) {
         if (pl.specials) {
@@ -531,6 +570,11 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
     pp.pay_in   = cur_pay;
     pp.pay_out  = dst_pay;
     pp.shift    = pass * RADIX_BITS;
+    {
+      uint8_t* side = pl.side_band ? reinterpret_cast<uint8_t*>(S + pl.off_digits) : nullptr;
+      pp.digits_in  = first ? nullptr : side;  // written by the pass before
+      pp.digits_out = last ? nullptr : side;   // read by the next upsweep, which runs after this scatter
+    }
     pp.slab_tot = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + (pass & 1) * pl.slab_tot_bytes);
     pp.slab_tot_next =
       last ? nullptr
@@ -1050,10 +1094,11 @@ int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int arg
   static const char* const pname[] = {"none", "idx32", "i64"};
   snprintf(buf, buf_bytes,
            "strategy=%s key_bytes=%d passes=%d digit_bits=%d tile=%d rows=%zu row_len=%zu "
-           "chunks_per_row=%zu tiles_per_chunk=%zu payload=%s specials=%d gather=%d scratch=%zu",
+           "chunks_per_row=%zu tiles_per_chunk=%zu payload=%s specials=%d gather=%d side_band=%d "
+           "scratch=%zu",
            sname[pl.strategy], pl.dt.bytes, pl.n_passes, RADIX_BITS, pl.tile, pl.rows, pl.row_len,
            pl.chunks_per_row, pl.tiles_per_chunk, pname[pl.pay], (int)pl.specials,
-           (int)pl.gather_values, pl.total);
+           (int)pl.gather_values, (int)pl.side_band, pl.total);
   return MISORT_OK;
 }
 

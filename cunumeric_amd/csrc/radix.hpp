@@ -65,6 +65,8 @@ __global__ void store_u64_kernel(unsigned long long* p, unsigned long long v) { 
 struct PassParams {
   const void* keys_in;   // FIRST: raw elements; else keys
   void* keys_out;        // LAST: raw elements (may be NULL when a payload is written); else keys
+  const uint8_t* digits_in;  // this pass's digit of every key of keys_in, or NULL (upsweep_digits_kernel)
+  uint8_t* digits_out;       // downsweep with SIDE: the NEXT pass's digit of every key written
   const void* pay_in;    // PAY_IDX32: u32 (ignored when FIRST); PAY_I64: int64, NULL => positions
   void* pay_out;         // PAY_IDX32: u32, int64 when LAST; PAY_I64: int64
   uint32_t* chunk_hist;             // [rows * chunks_per_row][RADIX] counts of this pass
@@ -234,6 +236,62 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
 }
 
 // ---------------------------------------------------------------------------------------
+// upsweep over the digit side-band.  A keys-only pass that is not the last also writes, for
+// every key it scatters, that key's digit for the NEXT pass as one byte (downsweep_kernel
+// with SIDE).  The next pass then counts those bytes instead of reading the keys again:
+// 1 byte per key instead of 4 or 8, and no key arithmetic.  Counters as in
+// count8_hist_kernel: every digit value has 32 counters, one per lane modulo 32 and in 32
+// different LDS banks, shared by the wavefronts of the workgroup, so the lanes of one atomic
+// never queue on a bank.
+// ---------------------------------------------------------------------------------------
+template <int NT>
+__global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
+{
+  constexpr int COPIES = 32;
+  __shared__ __attribute__((aligned(16))) uint32_t h[RADIX * COPIES];
+  for (int i = threadIdx.x; i < RADIX * COPIES; i += NT) h[i] = 0;
+  __syncthreads();
+  const uint32_t row   = blockIdx.x / p.chunks_per_row;
+  const uint32_t chunk = blockIdx.x % p.chunks_per_row;
+  const uint64_t clen  = (uint64_t)p.tiles_per_chunk * p.tile;
+  const uint64_t begin = (uint64_t)chunk * clen;
+  uint64_t end         = begin + clen;
+  if (end > p.row_len) end = p.row_len;
+  const uint64_t n    = end > begin ? end - begin : 0;
+  const uint8_t* base = p.digits_in + (uint64_t)row * p.row_len + begin;
+  uint32_t* my        = h + (threadIdx.x & (COPIES - 1));
+  auto count          = [&](uint32_t d) { atomicAdd(&my[d * COPIES], 1u); };
+
+  // bytes before the first 16-byte boundary and after the last one go one per thread
+  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15;
+  if (head > n) head = n;
+  const uint64_t nvec = (n - head) / 16;
+  const uint4* vbase  = reinterpret_cast<const uint4*>(base + head);
+  stream_vectors<4>(vbase, nvec, threadIdx.x, (uint32_t)NT, [&](const uint4& r) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      count(w[e] & 0xFFu);
+      count((w[e] >> 8) & 0xFFu);
+      count((w[e] >> 16) & 0xFFu);
+      count(w[e] >> 24);
+    }
+  });
+  const uint64_t tail0 = head + nvec * 16;
+  for (uint64_t i = threadIdx.x; i < head + (n - tail0); i += NT) count(base[i < head ? i : tail0 + (i - head)]);
+  __syncthreads();
+  uint32_t* out = p.chunk_hist + (uint64_t)blockIdx.x * RADIX;
+  unsigned long long* slab =
+    p.slab_tot + ((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX;
+  for (int d = threadIdx.x; d < RADIX; d += NT) {
+    uint32_t c = 0;
+    for (int i = 0; i < COPIES; ++i) c += h[d * COPIES + ((i + d) & (COPIES - 1))];  // rotated: no bank queue
+    out[d] = c;
+    if (c) atomicAdd(&slab[d], (unsigned long long)c);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // downsweep
 // ---------------------------------------------------------------------------------------
 // Loads one tile (wave-striped) into registers.  Slots past `valid` (partial last tile of
@@ -272,10 +330,21 @@ __device__ __forceinline__ void load_tile_payload(const PassParams& p, uint64_t 
 // value.  G elements of the narrowest array written are 128 bytes, capped so the carry
 // area stays within 64 KB.
 
+//
+// SIDE (keys-only passes that are not the last): the pass also writes the digit side-band,
+// the NEXT pass's digit of every key as one byte at the key's output position, for
+// upsweep_digits_kernel.  A digit run advances by a few dozen bytes of side-band per tile,
+// and a 128-byte line written in pieces that L2 evicts one by one costs as much as the
+// keys' whole lines, so the bytes have a carry of their own with 128 entries per digit value:
+// bytes of positions [brun, run) wait there (brun: start of the first line not yet
+// complete), and whenever the run passes a 128-byte boundary the waiting bytes and the new
+// ones up to that boundary go out together.
 template <typename KeyT, int PAY, bool FIRST, bool LAST, int NT, int IPT, int G, int OCC,
-          bool PART = false>
+          bool PART = false, bool SIDE = false>
 __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
 {
+  static_assert(!SIDE || (PAY == PAY_NONE && !LAST && !PART && (RADIX * G) / NT <= 8),
+                "the side-band is written by keys-only passes before the last");
   static_assert(NT % RADIX == 0 && (NT / 64) % (NT / RADIX) == 0, "whole groups of digit owners");
   static_assert((G & (G - 1)) == 0 && (RADIX * G) % NT == 0, "carry slots divide evenly");
   constexpr int NW   = NT / 64;
@@ -296,6 +365,17 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   __shared__ __attribute__((aligned(16))) PayT spay[PAY == PAY_NONE ? 1 : TILE];
   __shared__ __attribute__((aligned(16))) KeyT ckeys[RADIX * G];
   __shared__ __attribute__((aligned(16))) PayT cpay[PAY == PAY_NONE ? 1 : RADIX * G];
+  // side-band: byte carry (slot s of digit value d holds the byte of position brun + s) and,
+  // for the write-out of tile n-1, b_pos = brun before the tile and b_tab =
+  //   bits 0-7   how many waiting bytes go out (all of them, or 0),
+  //   bits 16-23 eb + 128: carried key e goes out directly if e < eb, else into byte-carry
+  //              slot e - eb.
+  // The same decision for staged slot q rides in dig_lim: (lim << 8) | delta, with q below
+  // lim - delta written directly and the rest of the written keys into slot q - (lim - delta).
+  constexpr int BL = 128;
+  __shared__ __attribute__((aligned(16))) uint8_t bcarry[SIDE ? RADIX * BL : 16];
+  __shared__ unsigned long long b_pos[SIDE ? RADIX : 1];
+  __shared__ uint32_t b_tab[SIDE ? RADIX : 1];
 
   const int tid        = threadIdx.x;
   const int lane       = tid & 63;
@@ -316,6 +396,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   // and how many elements of it wait in the carry
   unsigned long long run = 0;
   uint32_t carry_n       = 0;
+  unsigned long long brun = 0;  // SIDE: first position whose side-band byte is not yet written
 
   auto tile_valid = [&](uint32_t t) -> uint32_t {
     const uint64_t rem = p.row_len - (uint64_t)t * TILE;
@@ -411,6 +492,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
       tot += dig_oldk[w];
     }
     if (tid < RADIX) run = row_base + base + incl - total + before;
+    brun = run;
     // How a wave ranks its keys, chosen once per workgroup.  The cheap way is one returning LDS
     // add per key on the wave's counter of the key's digit value (1 LDS instruction instead of
     // 41 vector instructions).  It is stable only because the LDS of gfx950 serves those lanes
@@ -466,17 +548,45 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
       }
     }
 
+    uint32_t dfr[SIDE ? 8 : 1];  // SIDE: byte-carry writes of carried keys, held until the barrier
     if (has_prev) {
       // ---- carried elements whose line tile n-1 completes ----
       // thread x = tid + i*NT holds carry slot e = x % G of digit value x / G
       // All LDS reads of a batch are issued before the first store so that they overlap.
       constexpr int NB  = RADIX * G / NT;
       constexpr int BB  = NB < 8 ? NB : 8;
+      if constexpr (SIDE) {
+        // ---- side-band bytes whose line tile n-1 completes: thread x = tid + i*NT holds
+        // the four bytes w = x % 32 of digit value x / 32
+        constexpr int ND = RADIX * (BL / 4) / NT;
+        const uint32_t ft = fresh_tid();
+#pragma unroll
+        for (int i = 0; i < ND; ++i) {
+          const uint32_t x   = ft + i * NT;
+          const uint32_t d   = x / (BL / 4);
+          const uint32_t w4  = (x % (BL / 4)) * 4;
+          const uint32_t cnt = b_tab[d] & 0xFFu;
+          if (w4 < cnt) {
+            const uint32_t val           = reinterpret_cast<const uint32_t*>(bcarry)[x];
+            const unsigned long long pos = b_pos[d] + w4;
+            uint8_t* o                   = p.digits_out + pos;
+            if (cnt - w4 >= 4 && (pos & 3) == 0) {
+              *reinterpret_cast<uint32_t*>(o) = val;
+            } else {
+              o[0] = (uint8_t)val;
+              if (cnt - w4 > 1) o[1] = (uint8_t)(val >> 8);
+              if (cnt - w4 > 2) o[2] = (uint8_t)(val >> 16);
+              if (cnt - w4 > 3) o[3] = (uint8_t)(val >> 24);
+            }
+          }
+        }
+      }
       const uint32_t bt = fresh_tid();
       const uint32_t e  = bt % G;  // NT is a multiple of G
 #pragma unroll 1
       for (int i0 = 0; i0 < NB; i0 += BB) {
         uint32_t ok[BB];
+        uint32_t tb[SIDE ? BB : 1];
         unsigned long long orun[BB];
         KeyT bk[BB];
         PayT bv[PAY == PAY_NONE ? 1 : BB];
@@ -485,14 +595,28 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
           const uint32_t x = bt + (i0 + j) * NT;
           const uint32_t d = x / G;
           ok[j]            = dig_oldk[d];
+          if constexpr (SIDE) tb[j] = b_tab[d];
           orun[j]          = old_run[d];
           bk[j]            = ckeys[x];
           if (PAY != PAY_NONE) bv[j] = cpay[x];
         }
 #pragma unroll
         for (int j = 0; j < BB; ++j) {
-          if (e < ok[j])
+          if constexpr (SIDE) dfr[j] = ~0u;
+          if (e < ok[j]) {
             emit(orun[j] + e, bk[j], PAY == PAY_NONE ? PayT{} : bv[PAY == PAY_NONE ? 0 : j]);
+            if constexpr (SIDE) {
+              const int32_t eb = (int32_t)((tb[j] >> 16) & 0xFFu) - 128;
+              const uint32_t b = KeyOps<KeyT>::digit(bk[j], p.shift + RADIX_BITS);
+              if ((int32_t)e < eb) {
+                p.digits_out[orun[j] + e] = (uint8_t)b;
+              } else {
+                // into the byte carry, but only after the barrier: its old bytes are being read
+                const uint32_t d = (bt + (i0 + j) * NT) / G;
+                dfr[j]           = ((d * BL + (uint32_t)((int32_t)e - eb)) << 8) | b;
+              }
+            }
+          }
         }
       }
     }
@@ -521,16 +645,31 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
     // staged slots of tile n-1, from the registers filled before the barrier: to global
     // memory up to the line boundary of their digit value, the rest into the carry
     auto write_staged = [&]() {
+      if constexpr (SIDE) {
+        constexpr int NB = RADIX * G / NT;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          if (dfr[j] != ~0u) bcarry[dfr[j] >> 8] = (uint8_t)dfr[j];
+      }
 #pragma unroll
       for (int i = 0; i < IPT; ++i) {
         const uint32_t q = at + i * NT;
         const PayT v     = PAY == PAY_NONE ? PayT{} : av[PAY == PAY_NONE ? 0 : i];
+        const int32_t lim = SIDE ? (alim[i] >> 8) : alim[i];
         if (q < pvalid) {
-          if ((int32_t)q < alim[i]) {
+          if ((int32_t)q < lim) {
             emit(abase[i] + q, ak[i], v);
+            if constexpr (SIDE) {
+              const int32_t blim = lim - (alim[i] & 0xFF);
+              const uint32_t b   = KeyOps<KeyT>::digit(ak[i], p.shift + RADIX_BITS);
+              if ((int32_t)q < blim)
+                p.digits_out[abase[i] + q] = (uint8_t)b;
+              else
+                bcarry[digit_of(ak[i]) * BL + (uint32_t)((int32_t)q - blim)] = (uint8_t)b;
+            }
           } else {
             const uint32_t d = digit_of(ak[i]);
-            const uint32_t c = d * G + (uint32_t)((int32_t)q - alim[i]);
+            const uint32_t c = d * G + (uint32_t)((int32_t)q - lim);
             ckeys[c]         = ak[i];
             if (PAY != PAY_NONE) cpay[c] = v;
           }
@@ -660,7 +799,23 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
         const unsigned long long hi = (run + total) & ~(unsigned long long)(G - 1);
         const uint32_t flush        = more ? (hi > run ? (uint32_t)(hi - run) : 0u) : total;
         dig_base[dv] = run + carry_n - tile_start;
-        dig_lim[dv]  = (int32_t)(flush + tile_start) - (int32_t)carry_n;
+        const int32_t lim = (int32_t)(flush + tile_start) - (int32_t)carry_n;
+        if constexpr (SIDE) {
+          // the side-band goes out in whole 128-byte lines up to the new run position
+          // (everything at the end of the chunk); bytes of [brun, run) wait in the byte carry
+          const unsigned long long new_run = run + flush;
+          unsigned long long nb            = more ? (new_run & ~(unsigned long long)(BL - 1)) : new_run;
+          if (nb < brun) nb = brun;
+          const uint32_t cnt = nb > brun ? (uint32_t)(run - brun) : 0u;
+          long long eb       = (long long)nb - (long long)run;  // > -128
+          if (eb > 127) eb = 127;
+          b_pos[dv]   = brun;
+          b_tab[dv]   = cnt | ((uint32_t)(eb + 128) << 16);
+          dig_lim[dv] = (int32_t)(((uint32_t)lim << 8) | (uint32_t)(new_run - nb));
+          brun        = nb;
+        } else {
+          dig_lim[dv] = lim;
+        }
         dig_oldk[dv] = flush ? carry_n : 0u;
         old_run[dv]  = run;
         run += flush;

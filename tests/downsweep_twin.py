@@ -9,7 +9,11 @@ bounds-checked and the invariants the kernel depends on asserted:
     that has not been written out,
   * the carry index of an element lies in [0, G), the elements a step writes out are
     exactly the whole 128-byte groups, every output position is written exactly once,
-  * padding keys of a partial tile rank behind every real key and are never written.
+  * padding keys of a partial tile rank behind every real key and are never written,
+  * with ``side=True`` (the digit side-band of keys-only sorts: next to every key the pass
+    writes that key's digit for the NEXT pass as one byte, in whole 128-byte lines through a
+    second, 128-entry carry per digit value): every byte position is written exactly once,
+    a byte-carry slot lies in [0, 128) and is never overwritten while live.
 
 It restates what the scatter pass of CUB's DeviceRadixSort does for the reference
 (src/cunumeric/sort/cub_sort.cuh:60-71): a stable split of the row by one digit.
@@ -36,9 +40,14 @@ def chunk_bases(digits: np.ndarray, tile: int, tiles_per_chunk: int) -> np.ndarr
     return start[None, :] + before
 
 
-def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tiles_per_chunk: int):
+BLINE = 128  # bytes of the side-band written at a time
+
+
+def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tiles_per_chunk: int,
+              side: bool = False):
     """One pass over one row.  keys: unsigned keys; pay: payload array or None (positions are
-    synthesised).  Returns (keys_out, pay_out)."""
+    synthesised).  Returns (keys_out, pay_out), and with ``side`` also the side-band (the
+    next pass's digit of every key written, in output order)."""
     assert nt % RADIX == 0 and (RADIX * g) % nt == 0 and g & (g - 1) == 0
     n = keys.size
     nw, tile = nt // 64, nt * ipt
@@ -50,11 +59,19 @@ def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tile
     kout = np.zeros(n, dtype=keys.dtype)
     pout = np.zeros(n, dtype=np.int64)
     written = np.zeros(n, dtype=np.int32)
+    bout = np.zeros(n, dtype=np.uint8)
+    bwritten = np.zeros(n, dtype=np.int32)
+    next_digit = lambda k: (int(k) >> (shift + 8)) & (RADIX - 1)
 
     def emit(pos, k, v):
         assert 0 <= pos < n, f"output position {pos} outside the row"
         written[pos] += 1
         kout[pos], pout[pos] = k, v
+
+    def emit_byte(pos, b):
+        assert 0 <= pos < n, f"side-band position {pos} outside the row"
+        bwritten[pos] += 1
+        bout[pos] = b
 
     for chunk in range(bases.shape[0]):
         tile0 = chunk * tiles_per_chunk
@@ -72,6 +89,14 @@ def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tile
         ckeys = np.zeros(RADIX * g, dtype=keys.dtype)
         cpay = np.zeros(RADIX * g, dtype=np.int64)
         c_live = np.zeros(RADIX * g, dtype=bool)     # checker state
+        # side-band: owner registers and tables, byte carry
+        brun = run.copy()
+        b_cnt = np.zeros(RADIX, dtype=np.int64)
+        b_pos = np.zeros(RADIX, dtype=np.int64)
+        b_eb = np.zeros(RADIX, dtype=np.int64)
+        b_delta = np.zeros(RADIX, dtype=np.int64)
+        bcarry = np.zeros((RADIX, BLINE), dtype=np.uint8)
+        b_live = np.zeros((RADIX, BLINE), dtype=bool)
 
         for tno in range(tile0, tile_end + 1):       # the step after the last tile only writes out
             has_cur = tno < tile_end
@@ -80,6 +105,14 @@ def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tile
             pvalid = min(tile, n - (tno - 1) * tile) if has_prev else 0
             more = tno + 1 < tile_end
             if has_prev:
+                deferred = []   # byte-carry writes of carried keys: held back until the barrier
+                if side:
+                    # ---- side-band bytes whose 128-byte line tile n-1 completes
+                    for d in range(RADIX):
+                        for j in range(int(b_cnt[d])):
+                            assert b_live[d, j], f"byte-carry slot {j} of digit {d} flushed but empty"
+                            b_live[d, j] = False
+                            emit_byte(int(b_pos[d]) + j, bcarry[d, j])
                 # ---- carried elements whose group tile n-1 completes: thread x = tid + i*NT
                 # holds carry slot e = x % G of digit value x // G
                 for x in range(RADIX * g):
@@ -88,19 +121,40 @@ def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tile
                         assert c_live[x], f"carry slot {e} of digit {d} flushed but empty"
                         c_live[x] = False
                         emit(int(old_run[d]) + e, ckeys[x], cpay[x])
+                        if side:
+                            if e < b_eb[d]:
+                                emit_byte(int(old_run[d]) + e, next_digit(ckeys[x]))
+                            else:
+                                deferred.append((d, e - int(b_eb[d]), next_digit(ckeys[x])))
                 # ---- staged tile n-1 into registers (before the barrier) ...
                 staged = []
                 for q in range(tile):
                     ak = skeys[q]
                     d = digit_of(ak)
                     staged.append((q, ak, spay[q], d, int(dig_base[d]), int(dig_lim[d])))
-                # ---- ... then to global memory up to the group boundary, the rest to the carry
+                # ---- (barrier) ... then to global memory up to the group boundary, the rest
+                # to the carry
+                for d, slot, b in deferred:
+                    assert 0 <= slot < BLINE, f"byte-carry slot {slot} of digit {d} outside [0, {BLINE})"
+                    assert not b_live[d, slot], f"byte-carry slot {slot} of digit {d} overwritten while live"
+                    b_live[d, slot] = True
+                    bcarry[d, slot] = b
                 for q, ak, av, d, abase, alim in staged:
                     if q < pvalid:
                         assert s_live[q], f"staged slot {q} read but never written"
                         s_live[q] = False
                         if q < alim:
                             emit(abase + q, ak, av)
+                            if side:
+                                blim = alim - int(b_delta[d])
+                                if q < blim:
+                                    emit_byte(abase + q, next_digit(ak))
+                                else:
+                                    slot = q - blim
+                                    assert 0 <= slot < BLINE, f"byte-carry slot {slot} of digit {d} outside [0, {BLINE})"
+                                    assert not b_live[d, slot], f"byte-carry slot {slot} of digit {d} overwritten while live"
+                                    b_live[d, slot] = True
+                                    bcarry[d, slot] = next_digit(ak)
                         else:
                             e = q - alim
                             assert 0 <= e < g, f"carry index {e} of digit {d} outside [0, {g})"
@@ -149,6 +203,23 @@ def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tile
                 dig_lim[d] = flush + tile_start[d] - carry_n[d]
                 dig_oldk[d] = carry_n[d] if flush else 0
                 old_run[d] = run[d]
+                if side:
+                    # bytes of positions [brun, run) wait in the byte carry; whole lines up
+                    # to the new run position go out (everything at the end of the chunk)
+                    new_run = int(run[d]) + flush
+                    if more:
+                        nb = new_run & ~(BLINE - 1)
+                        new_brun = nb if nb > brun[d] else int(brun[d])
+                    else:
+                        new_brun = new_run
+                    assert int(run[d]) - int(brun[d]) < BLINE
+                    b_cnt[d] = int(run[d]) - int(brun[d]) if new_brun > brun[d] else 0
+                    assert b_cnt[d] == 0 or new_brun >= run[d], "a flushed byte carry is flushed whole"
+                    b_pos[d] = brun[d]
+                    b_eb[d] = new_brun - int(run[d])
+                    b_delta[d] = new_run - new_brun
+                    assert 0 <= b_delta[d] < BLINE or not more
+                    brun[d] = new_brun
                 run[d] += flush
                 carry_n[d] = total - flush
                 assert 0 <= carry_n[d] < g or not more, f"carry of digit {d} does not fit {g} slots"
@@ -170,5 +241,10 @@ def downsweep(keys: np.ndarray, pay, shift: int, nt: int, ipt: int, g: int, tile
                     s_live[q] = not pad[t, i]
         assert not s_live.any() and not c_live.any(), "elements left behind at the end of the chunk"
         assert (carry_n == 0).all()
+        assert not b_live.any(), "side-band bytes left behind at the end of the chunk"
+        assert not side or (brun == run).all()
     assert (written == 1).all(), "an output position was not written exactly once"
+    if side:
+        assert (bwritten == 1).all(), "a side-band position was not written exactly once"
+        return kout, pout, bout
     return kout, pout

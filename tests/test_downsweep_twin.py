@@ -70,3 +70,27 @@ def test_twin_kernel_geometry_with_payload(nt, ipt, g, dtype):
     ref_k, order = stable_split(keys, 8)
     assert np.array_equal(got_k, ref_k)
     assert np.array_equal(got_p, pay[order])
+
+
+@pytest.mark.parametrize("kind", ["uniform", "few", "const", "ones", "runs"])
+@pytest.mark.parametrize("nt,ipt,g,n,tpc", [
+    (256, 16, 32, 5 * 4096 + 77, 2),   # 4-byte keys only
+    (256, 7, 16, 9 * 1792 + 1, 4),     # 8-byte keys only
+    (256, 7, 16, 300, 4),              # a single partial tile
+    (512, 3, 16, 40 * 1536 + 5, 40),   # one chunk walks many tiles: lines complete every few steps
+    (256, 2, 16, 64 * 512 + 3, 16),    # two keys of a digit value per tile: the byte carry fills slowly
+])
+def test_twin_digit_side_band(kind, nt, ipt, g, n, tpc):
+    """Keys-only passes also write every key's digit for the next pass as a byte, in output
+    order, through the 128-entry byte carry: the bytes must be the next digit of the keys
+    where the pass put them, every position written once (asserted inside the twin)."""
+    dtype = np.uint64 if g <= 16 else np.uint32
+    rng = np.random.default_rng(hash((kind, nt, ipt, n, "side")) & 0xFFFF)
+    keys = make(kind, n, dtype, rng)
+    for shift in (0, 8 * (np.dtype(dtype).itemsize - 2)):
+        got_k, got_p, got_b = downsweep(keys, None, shift, nt, ipt, g, tpc, side=True)
+        ref_k, ref_p = stable_split(keys, shift)
+        assert np.array_equal(got_k, ref_k)
+        assert np.array_equal(got_p, ref_p)
+        nxt = (ref_k >> np.array(shift + 8, dtype)) & np.array(RADIX - 1, dtype)
+        assert np.array_equal(got_b, nxt.astype(np.uint8))
