@@ -229,7 +229,10 @@ struct Plan {
   // digit side-band of keys-only sorts: one byte per key, written by every pass but the last
   // and counted by the next pass's upsweep in place of the keys
   bool side_band = false;
-  size_t off_digits = 0;
+  // the other radix sorts of 4-byte and wider keys: a pass writes the side-band, without the
+  // byte carry, only where few digit values are in use; it says so per row in side_flag
+  bool side_adaptive = false;
+  size_t off_digits = 0, off_side_flag = 0;
   size_t off_gather_idx = 0, off_gather_src = 0;
   // counting sort of 2-byte keys: chunks of the histogram kernel, counters, their scan
   size_t c16_chunks = 0, c16_chunk_len = 0, off_c16_hist = 0, off_c16_prefix = 0;
@@ -344,6 +347,7 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.slab_tot_bytes    = pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long);
     pl.off_slab_tot      = take(pl.slab_tot_bytes);
     take(pl.slab_tot_bytes);
+    pl.off_side_flag     = take(2 * pl.rows * sizeof(uint32_t));  // per pass parity and row
     pl.zero_bytes        = off - pl.off_special_ctr;
     pl.off_chunk_hist    = take(pl.n_chunks * RADIX * sizeof(uint32_t));
 
@@ -362,7 +366,9 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // (8-byte keys: the upsweep saves 7 of 8 bytes per key; with 4-byte keys the extra
     // stores of the scatter cost more than the upsweep saves)
     pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
-    if (pl.side_band) pl.off_digits = take(pl.volume);
+    pl.side_adaptive = side_band_default() && !pl.side_band && pl.n_passes >= 2 && pl.dt.bytes >= 4 &&
+                       (pl.pay != PAY_NONE || pl.dt.bytes > 4);
+    if (pl.side_band || pl.side_adaptive) pl.off_digits = take(pl.volume);
     if (pl.specials)
       pl.off_special_blk =
         take(pl.n_chunks * (kUpsweepThreads / 64) * 2 * sizeof(unsigned long long));
@@ -466,7 +472,7 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
   const dim3 grid((unsigned)pl.n_chunks);
 
   L.run(K_UPSWEEP, [&] {
-    if (pp.digits_in) {
+    if (pp.digits_in && !pp.side_flag_in) {  // the pass before always writes the side-band
       hipLaunchKernelGGL((upsweep_digits_kernel<kUpsweepDigitThreads>), grid, dim3(kUpsweepDigitThreads), 0,
                          L.stream, pp);
       return;
@@ -571,9 +577,12 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
     pp.pay_out  = dst_pay;
     pp.shift    = pass * RADIX_BITS;
     {
-      uint8_t* side = pl.side_band ? reinterpret_cast<uint8_t*>(S + pl.off_digits) : nullptr;
+      uint8_t* side = (pl.side_band || pl.side_adaptive) ? reinterpret_cast<uint8_t*>(S + pl.off_digits) : nullptr;
       pp.digits_in  = first ? nullptr : side;  // written by the pass before
       pp.digits_out = last ? nullptr : side;   // read by the next upsweep, which runs after this scatter
+      uint32_t* flag   = reinterpret_cast<uint32_t*>(S + pl.off_side_flag);
+      pp.side_flag_in  = (pl.side_adaptive && !first) ? flag + ((pass - 1) & 1) * pl.rows : nullptr;
+      pp.side_flag_out = (pl.side_adaptive && !last) ? flag + (pass & 1) * pl.rows : nullptr;
     }
     pp.slab_tot = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + (pass & 1) * pl.slab_tot_bytes);
     pp.slab_tot_next =
@@ -1098,7 +1107,7 @@ int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int arg
            "scratch=%zu",
            sname[pl.strategy], pl.dt.bytes, pl.n_passes, RADIX_BITS, pl.tile, pl.rows, pl.row_len,
            pl.chunks_per_row, pl.tiles_per_chunk, pname[pl.pay], (int)pl.specials,
-           (int)pl.gather_values, (int)pl.side_band, pl.total);
+           (int)pl.gather_values, pl.side_band ? 1 : (pl.side_adaptive ? 2 : 0), pl.total);
   return MISORT_OK;
 }
 

@@ -69,7 +69,10 @@ struct PassParams {
   const void* keys_in;   // FIRST: raw elements; else keys
   void* keys_out;        // LAST: raw elements (may be NULL when a payload is written); else keys
   const uint8_t* digits_in;  // this pass's digit of every key of keys_in, or NULL (upsweep_digits_kernel)
-  uint8_t* digits_out;       // downsweep with SIDE: the NEXT pass's digit of every key written
+  uint8_t* digits_out;       // downsweep: the NEXT pass's digit of every key written (always with
+                             // SIDE, otherwise only where the pass decides that it pays), or NULL
+  const uint32_t* side_flag_in;  // [rows] 1 where the pass before wrote digits_in for the row, or NULL
+  uint32_t* side_flag_out;       // [rows] where this pass says whether it writes digits_out, or NULL
   const void* pay_in;    // PAY_IDX32: u32 (ignored when FIRST); PAY_I64: int64, NULL => positions
   void* pay_out;         // PAY_IDX32: u32, int64 when LAST; PAY_I64: int64
   uint32_t* chunk_hist;             // [rows * chunks_per_row][RADIX] counts of this pass
@@ -120,6 +123,14 @@ __device__ __forceinline__ void pin_value(T& v)
   }
 }
 
+// A pass without a byte carry writes the digit side-band only if a tile of the row holds at
+// most this many digit values on average (random digits: 256, where it costs 0.4 ms per pass
+// at 2^28 keys and saves 0.15-0.3 ms in the next upsweep).
+#ifndef MISORT_SIDE_PRESENT_MAX
+#define MISORT_SIDE_PRESENT_MAX 64
+#endif
+static constexpr uint32_t kSidePresentMax = MISORT_SIDE_PRESENT_MAX;
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load and store of the wave, which would serialise the prefetch of the
 // next tile and the draining stores of the previous one with the arithmetic in between.
@@ -128,6 +139,68 @@ __device__ __forceinline__ void lds_barrier()
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// ---------------------------------------------------------------------------------------
+// upsweep over the digit side-band.  A keys-only pass that is not the last also writes, for
+// every key it scatters, that key's digit for the NEXT pass as one byte (downsweep_kernel
+// with SIDE).  The next pass then counts those bytes instead of reading the keys again:
+// 1 byte per key instead of 4 or 8, and no key arithmetic.  Counters as in
+// count8_hist_kernel: every digit value has 32 counters, one per lane modulo 32 and in 32
+// different LDS banks, shared by the wavefronts of the workgroup, so the lanes of one atomic
+// never queue on a bank.
+// ---------------------------------------------------------------------------------------
+template <int NT>
+__device__ __forceinline__ void count_digit_bytes(const PassParams& p, uint32_t* h /* LDS, RADIX * 32 words */)
+{
+  constexpr int COPIES = 32;
+  for (int i = threadIdx.x; i < RADIX * COPIES; i += NT) h[i] = 0;
+  __syncthreads();
+  const uint32_t row   = blockIdx.x / p.chunks_per_row;
+  const uint32_t chunk = blockIdx.x % p.chunks_per_row;
+  const uint64_t clen  = (uint64_t)p.tiles_per_chunk * p.tile;
+  const uint64_t begin = (uint64_t)chunk * clen;
+  uint64_t end         = begin + clen;
+  if (end > p.row_len) end = p.row_len;
+  const uint64_t n    = end > begin ? end - begin : 0;
+  const uint8_t* base = p.digits_in + (uint64_t)row * p.row_len + begin;
+  uint32_t* my        = h + (threadIdx.x & (COPIES - 1));
+  auto count          = [&](uint32_t d) { atomicAdd(&my[d * COPIES], 1u); };
+
+  // bytes before the first 16-byte boundary and after the last one go one per thread
+  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15;
+  if (head > n) head = n;
+  const uint64_t nvec = (n - head) / 16;
+  const uint4* vbase  = reinterpret_cast<const uint4*>(base + head);
+  stream_vectors<4>(vbase, nvec, threadIdx.x, (uint32_t)NT, [&](const uint4& r) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      count(w[e] & 0xFFu);
+      count((w[e] >> 8) & 0xFFu);
+      count((w[e] >> 16) & 0xFFu);
+      count(w[e] >> 24);
+    }
+  });
+  const uint64_t tail0 = head + nvec * 16;
+  for (uint64_t i = threadIdx.x; i < head + (n - tail0); i += NT) count(base[i < head ? i : tail0 + (i - head)]);
+  __syncthreads();
+  uint32_t* out = p.chunk_hist + (uint64_t)blockIdx.x * RADIX;
+  unsigned long long* slab =
+    p.slab_tot + ((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX;
+  for (int d = threadIdx.x; d < RADIX; d += NT) {
+    uint32_t c = 0;
+    for (int i = 0; i < COPIES; ++i) c += h[d * COPIES + ((i + d) & (COPIES - 1))];  // rotated: no bank queue
+    out[d] = c;
+    if (c) atomicAdd(&slab[d], (unsigned long long)c);
+  }
+}
+
+template <int NT>
+__global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
+{
+  __shared__ __attribute__((aligned(16))) uint32_t h[RADIX * 32];
+  count_digit_bytes<NT>(p, h);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -143,12 +216,20 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   // (different LDS banks): when a few digit values dominate, lanes that would queue up on
   // one counter are spread over four.
   constexpr int COPIES = 4;
-  __shared__ __attribute__((aligned(16))) uint32_t lhist[NW * RADIX * COPIES];
+  constexpr int WORDS  = NW * RADIX * COPIES > RADIX * 32 ? NW * RADIX * COPIES : RADIX * 32;
+  __shared__ __attribute__((aligned(16))) uint32_t lhist[WORDS];
+  const uint32_t row   = blockIdx.x / p.chunks_per_row;
+  const uint32_t chunk = blockIdx.x % p.chunks_per_row;
+  if constexpr (!FIRST && !SPECIALS && !PART) {
+    // the pass before wrote this pass's digits as bytes for this row: count those
+    if (p.side_flag_in && p.side_flag_in[row]) {
+      count_digit_bytes<NT>(p, lhist);
+      return;
+    }
+  }
   for (int i = threadIdx.x; i < NW * RADIX * COPIES; i += NT) lhist[i] = 0;
   __syncthreads();
 
-  const uint32_t row   = blockIdx.x / p.chunks_per_row;
-  const uint32_t chunk = blockIdx.x % p.chunks_per_row;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const KeyT* in        = reinterpret_cast<const KeyT*>(p.keys_in) + (uint64_t)row * p.row_len;
   const uint64_t clen   = (uint64_t)p.tiles_per_chunk * p.tile;
@@ -233,62 +314,6 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       const uint4 q = *reinterpret_cast<const uint4*>(&lhist[(w * RADIX + d) * COPIES]);
       c += q.x + q.y + q.z + q.w;
     }
-    out[d] = c;
-    if (c) atomicAdd(&slab[d], (unsigned long long)c);
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// upsweep over the digit side-band.  A keys-only pass that is not the last also writes, for
-// every key it scatters, that key's digit for the NEXT pass as one byte (downsweep_kernel
-// with SIDE).  The next pass then counts those bytes instead of reading the keys again:
-// 1 byte per key instead of 4 or 8, and no key arithmetic.  Counters as in
-// count8_hist_kernel: every digit value has 32 counters, one per lane modulo 32 and in 32
-// different LDS banks, shared by the wavefronts of the workgroup, so the lanes of one atomic
-// never queue on a bank.
-// ---------------------------------------------------------------------------------------
-template <int NT>
-__global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
-{
-  constexpr int COPIES = 32;
-  __shared__ __attribute__((aligned(16))) uint32_t h[RADIX * COPIES];
-  for (int i = threadIdx.x; i < RADIX * COPIES; i += NT) h[i] = 0;
-  __syncthreads();
-  const uint32_t row   = blockIdx.x / p.chunks_per_row;
-  const uint32_t chunk = blockIdx.x % p.chunks_per_row;
-  const uint64_t clen  = (uint64_t)p.tiles_per_chunk * p.tile;
-  const uint64_t begin = (uint64_t)chunk * clen;
-  uint64_t end         = begin + clen;
-  if (end > p.row_len) end = p.row_len;
-  const uint64_t n    = end > begin ? end - begin : 0;
-  const uint8_t* base = p.digits_in + (uint64_t)row * p.row_len + begin;
-  uint32_t* my        = h + (threadIdx.x & (COPIES - 1));
-  auto count          = [&](uint32_t d) { atomicAdd(&my[d * COPIES], 1u); };
-
-  // bytes before the first 16-byte boundary and after the last one go one per thread
-  uint64_t head = (16 - (reinterpret_cast<uintptr_t>(base) & 15)) & 15;
-  if (head > n) head = n;
-  const uint64_t nvec = (n - head) / 16;
-  const uint4* vbase  = reinterpret_cast<const uint4*>(base + head);
-  stream_vectors<4>(vbase, nvec, threadIdx.x, (uint32_t)NT, [&](const uint4& r) {
-    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      count(w[e] & 0xFFu);
-      count((w[e] >> 8) & 0xFFu);
-      count((w[e] >> 16) & 0xFFu);
-      count(w[e] >> 24);
-    }
-  });
-  const uint64_t tail0 = head + nvec * 16;
-  for (uint64_t i = threadIdx.x; i < head + (n - tail0); i += NT) count(base[i < head ? i : tail0 + (i - head)]);
-  __syncthreads();
-  uint32_t* out = p.chunk_hist + (uint64_t)blockIdx.x * RADIX;
-  unsigned long long* slab =
-    p.slab_tot + ((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX;
-  for (int d = threadIdx.x; d < RADIX; d += NT) {
-    uint32_t c = 0;
-    for (int i = 0; i < COPIES; ++i) c += h[d * COPIES + ((i + d) & (COPIES - 1))];  // rotated: no bank queue
     out[d] = c;
     if (c) atomicAdd(&slab[d], (unsigned long long)c);
   }
@@ -406,12 +431,21 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
     return rem < (uint64_t)TILE ? (uint32_t)rem : (uint32_t)TILE;
   };
 
+  // Without SIDE (sorts with a payload, 16-byte keys): whether this pass writes the side-band
+  // anyway, byte by byte next to the keys.  That costs a partly written 128-byte line per digit
+  // value and tile, so it pays only where few digit values are in use (long runs per tile);
+  // decided below from the row's counts, the same way by every workgroup of the row.
+  constexpr bool ADAPT = !SIDE && !PART && !LAST && sizeof(KeyT) >= 4 && (PAY != PAY_NONE || sizeof(KeyT) > 4);
+  bool side_on = false;
   KeyT* kout = reinterpret_cast<KeyT*>(p.keys_out);
   auto emit  = [&](unsigned long long dst, KeyT k, PayT v) {
     if (LAST) {
       if (kout) kout[dst] = KeyOps<KeyT>::from_key(k, p.xform);
     } else {
       kout[dst] = k;
+      if constexpr (ADAPT) {
+        if (side_on) p.digits_out[dst] = (uint8_t)KeyOps<KeyT>::digit(k, p.shift + RADIX_BITS);
+      }
     }
     if (PAY == PAY_IDX32) {
       if (LAST)
@@ -480,19 +514,37 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
       m = max(m, (uint32_t)__shfl_xor((int)m, s, 64));
       c += (uint32_t)__shfl_xor((int)c, s, 64);
     }
+    // how many digit values a tile of this row holds on average, in 1/65536: a value with
+    // count c is in a tile with probability min(1, c * TILE / row_len)
+    uint32_t present = 0;
+    if (tid < RADIX) {
+      const unsigned long long t = total * (unsigned long long)TILE;
+      present = t >= p.row_len ? 65536u : (uint32_t)((t << 16) / p.row_len);
+    }
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) present += (uint32_t)__shfl_xor((int)present, s, 64);
     if (lane == 63 && wave < RADIX / 64) {
       old_run[wave]  = incl;
       dig_lim[wave]  = (int32_t)m;
       dig_oldk[wave] = c;
+      dig_base[wave] = present;
     }
     __syncthreads();
     unsigned long long base = 0;
     uint32_t mx = 0, tot = 0;
+    present = 0;
 #pragma unroll
     for (int w = 0; w < RADIX / 64; ++w) {
       if (w < wave) base += old_run[w];
       mx = max(mx, (uint32_t)dig_lim[w]);
       tot += dig_oldk[w];
+      present += (uint32_t)dig_base[w];
+    }
+    if constexpr (ADAPT) {
+      if (p.digits_out) {
+        side_on = __builtin_amdgcn_readfirstlane((int)(present <= kSidePresentMax * 65536u)) != 0;
+        if (chunk == 0 && tid == 0 && p.side_flag_out) p.side_flag_out[row] = side_on ? 1u : 0u;
+      }
     }
     if (tid < RADIX) run = row_base + base + incl - total + before;
     brun = run;

@@ -92,3 +92,60 @@ def test_switch_off_gives_the_same_result():
         outs.append(r.stdout.strip().splitlines())
     assert outs[0][-1] == "True" and outs[1][-1] == "True"
     assert "side_band=1" in outs[0][0] and "side_band=0" in outs[1][0]
+
+
+# ---- sorts with positions (and 16-byte keys): a pass writes the side-band, without the byte
+# carry, only for rows in which few digit values are in use, and says so per row ----
+
+def few_values(dtype, n, rng, k=16):
+    dt = np.dtype(dtype)
+    if dt.kind in "iu":
+        ii = np.iinfo(dt)
+        vals = rng.integers(ii.min, ii.max, k, dtype=dt, endpoint=True)
+    elif dt.kind == "c":
+        vals = (rng.standard_normal(k) + 1j * rng.standard_normal(k)).astype(dt)
+    else:
+        vals = rng.standard_normal(k).astype(dt)
+    w = np.arange(1, k + 1, dtype=np.float64) ** -1.2
+    return vals[rng.choice(k, n, p=w / w.sum())]
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64, np.float64, np.complex64, np.complex128],
+                         ids=lambda d: np.dtype(d).name)
+def test_argsort_few_digit_values(abi, dtype):
+    rng = np.random.default_rng(51)
+    n = (1 << 20) + 4321
+    inputs = {"16 values": few_values(dtype, n, rng), "3 values": few_values(dtype, n, rng, 3)}
+    if np.dtype(dtype).kind in "iu":
+        inputs["small range"] = rng.integers(0, 200, n).astype(dtype)   # upper digits all equal
+    for name, a in inputs.items():
+        for chunks in (0, 5):
+            print(f"adaptive side-band dtype={np.dtype(dtype).name} case={name} chunks={chunks}", flush=True)
+            got = abi.local_sort(a, n, argsort=True, chunks=chunks)
+            assert np.array_equal(got, np.argsort(a, kind="stable")), (name, chunks)
+    if np.dtype(dtype).kind == "c":   # 16-byte keys (complex128) and complex64 also sort values through positions
+        a = inputs["16 values"]
+        assert bits_equal(abi.local_sort(a, n, argsort=False), np.sort(a, kind="stable"))
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float64], ids=lambda d: np.dtype(d).name)
+def test_rows_that_decide_differently(abi, dtype):
+    """Rows with few values, a constant row and random rows in one call: every row decides
+    for itself in every pass, and the next upsweep must follow each row's own flag."""
+    rng = np.random.default_rng(52)
+    rows, row_len = 6, 150001
+    a = np.empty((rows, row_len), dtype=dtype)
+    a[0] = few_values(dtype, row_len, rng)
+    a[1] = random_array(dtype, row_len, rng)
+    a[2] = np.full(row_len, a[1, 0], dtype=dtype)
+    a[3] = random_array(dtype, row_len, rng, narrow=True)
+    a[4] = random_array(dtype, row_len, rng)
+    a[5] = few_values(dtype, row_len, rng, 40)
+    for chunks in (rows, 4 * rows):
+        print(f"adaptive side-band rows dtype={np.dtype(dtype).name} chunks={chunks}", flush=True)
+        got = abi.local_sort(a, row_len, argsort=True, chunks=chunks).reshape(rows, row_len)
+        assert np.array_equal(got, np.argsort(a, axis=1, kind="stable"))
+    pay = rng.integers(-(2**62), 2**62, rows * row_len, dtype=np.int64)
+    got = abi.local_sort(a, row_len, argsort=True, indices_in=pay, chunks=2 * rows).reshape(rows, row_len)
+    ref = np.take_along_axis(pay.reshape(rows, row_len), np.argsort(a, axis=1, kind="stable"), axis=1)
+    assert np.array_equal(got, ref)
