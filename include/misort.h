@@ -75,6 +75,10 @@ const char* misort_last_error(void);
  * storage (src/cunumeric/sort/cub_sort.cuh:60-62) and the key / index staging
  * buffers it allocates from the Legate pool (cub_sort.cuh:46-52, 110-116;
  * sort.cu:1698).  Returns 0 when volume == 0.
+ * The radix path of 4-byte and wider keys includes one byte per element for a digit
+ * side-band (each pass can leave the next pass's digit of every key there, so that the next
+ * count reads bytes instead of keys); MISORT_SIDE_BAND=0 in the environment before the first
+ * call into the library leaves it out (give the query and the sort the same environment).
  */
 size_t misort_scratch_bytes(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                             int has_indices_in);
