@@ -28,6 +28,8 @@ EXPORTS = (
     "misort_local_static",
     "misort_selftest_lds_lane_order",
     "misort_searchsorted",
+    "misort_searchsorted_scratch_bytes",
+    "misort_searchsorted_ws",
     "misort_unique_scratch_bytes",
     "misort_unique",
     "misort_partition_scratch_bytes",
@@ -101,6 +103,11 @@ def load():
     lib.misort_kernel_name.argtypes = [c_int]
     lib.misort_describe_plan.restype = c_int
     lib.misort_describe_plan.argtypes = [c_int, c_size_t, c_size_t, c_int, c_int, c_char_p, c_size_t]
+    lib.misort_searchsorted_scratch_bytes.restype = c_size_t
+    lib.misort_searchsorted_scratch_bytes.argtypes = [c_int, c_size_t, c_size_t]
+    lib.misort_searchsorted_ws.restype = c_int
+    lib.misort_searchsorted_ws.argtypes = [c_int, c_void_p, c_size_t, c_void_p, c_size_t, c_int, c_void_p,
+                                           c_void_p, c_size_t, c_void_p]
     lib.misort_searchsorted.restype = c_int
     lib.misort_searchsorted.argtypes = [c_int, c_void_p, c_size_t, c_void_p, c_size_t, c_int, c_void_p,
                                         c_void_p]

@@ -295,10 +295,16 @@ class ndarray:
         v_ndarray = queries
         result = ndarray(v_ndarray.shape, np.int64)
         if v_ndarray.size:
+            lib = _lib.load()
+            code = to_core_dtype(a.dtype)
+            # many queries into a large array: the library sorts the queries first (workspace)
+            need = lib.misort_searchsorted_scratch_bytes(code, a.size, v_ndarray.size)
+            scratch = runtime.alloc_bytes(need) if need else None
             _lib.check(
-                _lib.load().misort_searchsorted(
-                    to_core_dtype(a.dtype), a._ptr() if a.size else None, a.size, v_ndarray._ptr(),
-                    v_ndarray.size, int(side == "left"), result._ptr(), runtime.stream_handle(),
+                lib.misort_searchsorted_ws(
+                    code, a._ptr() if a.size else None, a.size, v_ndarray._ptr(), v_ndarray.size,
+                    int(side == "left"), result._ptr(), scratch.data_ptr() if need else None, need,
+                    runtime.stream_handle(),
                 )
             )
         if scalar:

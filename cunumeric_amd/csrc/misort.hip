@@ -858,7 +858,7 @@ static void partition_select_pay(Launcher& L, const PartLayout& u, const void* v
 static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_out,
                     const int64_t* indices_in, int64_t* indices_out, size_t volume,
                     size_t sort_dim_size, int64_t index_offset, void* scratch, size_t scratch_bytes,
-                    size_t target_chunks = 0)
+                    size_t target_chunks = 0, bool canonical_values = false)
 {
   Plan pl;
   const bool argsort = indices_out != nullptr;
@@ -904,7 +904,11 @@ static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_
   // (With a caller-filled payload there are no positions to gather by: the last pass
   // writes the keys back through the inverse transform instead.)
   SortArgs core = a;
-  const bool gather_sorted = argsort && values_out && !indices_in;
+  // (canonical_values: the caller only compares the sorted values through their keys, so the
+  // last pass may write them through the inverse key transform, which maps -0 to +0 and
+  // every NaN to one NaN; not for complex elements, whose NaN tiers have no inverse)
+  const bool gather_sorted =
+    argsort && values_out && !indices_in && !(canonical_values && pl.dt.xform != XF_COMPLEX);
   if (gather_sorted) core.values_out = nullptr;
   if (argsort && values_out && indices_in && pl.dt.xform == XF_COMPLEX)
     return fail(MISORT_ERR_UNSUPPORTED,
@@ -1111,8 +1115,41 @@ int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int arg
   return MISORT_OK;
 }
 
-int misort_searchsorted(int dtype, const void* sorted, size_t n, const void* values, size_t m,
-                        int left, int64_t* out, void* stream)
+// searchsorted with the queries sorted first: [sorted queries | their positions | scratch of the sort]
+struct SearchLayout {
+  size_t off_pos = 0, off_sort = 0, sort_bytes = 0, total = 0;
+};
+// Sorting the queries pays when there are many of them and the array is larger than the
+// caches.  Measured with float32, plain / sorted first: 2^28 elements, 2^24 queries 3.81 /
+// 1.18 ms, 2^20 queries 0.34 / 0.33 ms, 2^19 queries 0.15 / 0.29 ms; 2^24 elements, 2^20
+// queries 0.19 / 0.11 ms.
+static bool search_sorts_queries(size_t elem_bytes, size_t n, size_t m)
+{
+  return m >= ((size_t)1 << 20) && n * elem_bytes >= ((size_t)64 << 20);
+}
+static bool search_layout(int dtype, size_t m, SearchLayout& u)
+{
+  DtypeInfo dt;
+  if (!dtype_info(dtype, dt)) return false;
+  Plan pl;
+  if (make_plan(dtype, m, m, true, false, pl) != MISORT_OK) return false;
+  u.off_pos    = align_up(m * dt.bytes, 256);
+  u.off_sort   = u.off_pos + align_up(m * sizeof(int64_t), 256);
+  u.sort_bytes = pl.total;
+  u.total      = u.off_sort + align_up(pl.total, 256) + 256;
+  return true;
+}
+
+size_t misort_searchsorted_scratch_bytes(int dtype, size_t n, size_t m)
+{
+  DtypeInfo dt;
+  if (!dtype_info(dtype, dt) || !search_sorts_queries(dt.bytes, n, m)) return 0;
+  SearchLayout u;
+  return search_layout(dtype, m, u) ? u.total : 0;
+}
+
+int misort_searchsorted_ws(int dtype, const void* sorted, size_t n, const void* values, size_t m,
+                           int left, int64_t* out, void* scratch, size_t scratch_bytes, void* stream)
 {
   DtypeInfo dt;
   if (!dtype_info(dtype, dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
@@ -1122,26 +1159,69 @@ int misort_searchsorted(int dtype, const void* sorted, size_t n, const void* val
   if (misaligned(values, dt.bytes) || (n != 0 && misaligned(sorted, dt.bytes)) || misaligned(out, 8))
     return fail(MISORT_ERR_ALIGN, "searchsorted: pointer not aligned to its element size");
   Launcher L;
-  L.stream      = reinterpret_cast<hipStream_t>(stream);
-  size_t blocks = (m + SEARCH_NT - 1) / SEARCH_NT;
-  if (blocks > 1024) blocks = 1024;
-  L.run(K_SEARCHSORTED, [&] {
+  L.stream = reinterpret_cast<hipStream_t>(stream);
+  const void* queries  = values;
+  const int64_t* where = nullptr;
+  if (scratch && search_sorts_queries(dt.bytes, n, m)) {
+    SearchLayout u;
+    if (!search_layout(dtype, m, u)) return fail(MISORT_ERR_UNSUPPORTED, "searchsorted: cannot plan the sort");
+    if (scratch_bytes < u.total) return fail(MISORT_ERR_SCRATCH, "searchsorted: scratch too small");
+    if (misaligned(scratch, 256)) return fail(MISORT_ERR_ALIGN, "scratch not aligned to 256 bytes");
+    char* S      = reinterpret_cast<char*>(scratch);
+    int64_t* pos = reinterpret_cast<int64_t*>(S + u.off_pos);
+    const int rc = run_sort(L, dtype, values, S, nullptr, pos, m, m, 0, S + u.off_sort,
+                            u.sort_bytes > 0 ? u.sort_bytes : 256, 0, true);
+    if (rc != MISORT_OK) return rc;
+    queries = S;
+    where   = pos;
+  }
+  if (where) {
+    // consecutive sorted queries per workgroup; about 2048 workgroups
+    size_t per_block = (m + 2047) / 2048;
+    per_block        = (per_block + SEARCH_NT - 1) / SEARCH_NT * SEARCH_NT;
+    const size_t blocks = (m + per_block - 1) / per_block;
+    L.run(K_SEARCHSORTED, [&] {
+#define MISORT_SEARCH_CASE(RAW)                                                                    \
+  hipLaunchKernelGGL((searchsorted_sorted_kernel<RAW>), dim3((unsigned)blocks), dim3(SEARCH_NT), 0, \
+                     L.stream, reinterpret_cast<const RAW*>(sorted), (uint64_t)n,                 \
+                     reinterpret_cast<const RAW*>(queries), (uint64_t)m, dt.xform, left, out, where, \
+                     (uint64_t)per_block)
+      switch (dt.bytes) {
+        case 1: MISORT_SEARCH_CASE(uint8_t); break;
+        case 2: MISORT_SEARCH_CASE(uint16_t); break;
+        case 4: MISORT_SEARCH_CASE(uint32_t); break;
+        case 8: MISORT_SEARCH_CASE(uint64_t); break;
+        default: MISORT_SEARCH_CASE(u128); break;
+      }
+#undef MISORT_SEARCH_CASE
+    });
+  } else {
+    size_t blocks = (m + SEARCH_NT - 1) / SEARCH_NT;
+    if (blocks > 1024) blocks = 1024;
+    L.run(K_SEARCHSORTED, [&] {
 #define MISORT_SEARCH_CASE(RAW)                                                                    \
   hipLaunchKernelGGL((searchsorted_kernel<RAW>), dim3((unsigned)blocks), dim3(SEARCH_NT), 0, L.stream, \
                      reinterpret_cast<const RAW*>(sorted), (uint64_t)n,                           \
-                     reinterpret_cast<const RAW*>(values), (uint64_t)m, dt.xform, left, out)
-    switch (dt.bytes) {
-      case 1: MISORT_SEARCH_CASE(uint8_t); break;
-      case 2: MISORT_SEARCH_CASE(uint16_t); break;
-      case 4: MISORT_SEARCH_CASE(uint32_t); break;
-      case 8: MISORT_SEARCH_CASE(uint64_t); break;
-      default: MISORT_SEARCH_CASE(u128); break;
-    }
+                     reinterpret_cast<const RAW*>(queries), (uint64_t)m, dt.xform, left, out)
+      switch (dt.bytes) {
+        case 1: MISORT_SEARCH_CASE(uint8_t); break;
+        case 2: MISORT_SEARCH_CASE(uint16_t); break;
+        case 4: MISORT_SEARCH_CASE(uint32_t); break;
+        case 8: MISORT_SEARCH_CASE(uint64_t); break;
+        default: MISORT_SEARCH_CASE(u128); break;
+      }
 #undef MISORT_SEARCH_CASE
-  });
+    });
+  }
   if (L.err != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
   return MISORT_OK;
+}
+
+int misort_searchsorted(int dtype, const void* sorted, size_t n, const void* values, size_t m,
+                        int left, int64_t* out, void* stream)
+{
+  return misort_searchsorted_ws(dtype, sorted, n, values, m, left, out, nullptr, 0, stream);
 }
 
 // scratch of misort_unique: [sorted copy | per-block counts | scratch of the sort]

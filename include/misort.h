@@ -145,6 +145,20 @@ int misort_searchsorted(int dtype, const void* sorted, size_t n, const void* val
                         int left, int64_t* out, void* stream);
 
 /*
+ * misort_searchsorted with a workspace.  Many random queries into an array far larger than
+ * the caches spend their time fetching one cache line per probe; with a workspace the queries
+ * are sorted first (by this library, with their positions), so that neighbouring threads
+ * probe neighbouring elements, and every answer is stored at the position its query came
+ * from.  misort_searchsorted_scratch_bytes returns 0 where that does not pay (few queries or
+ * a small array); scratch may then be NULL and the call is misort_searchsorted.  No
+ * counterpart in the reference (one cub::LowerBound / UpperBound per query,
+ * src/cunumeric/sort/searchsorted.cu:25-63).
+ */
+size_t misort_searchsorted_scratch_bytes(int dtype, size_t n, size_t m);
+int misort_searchsorted_ws(int dtype, const void* sorted, size_t n, const void* values, size_t m,
+                           int left, int64_t* out, void* scratch, size_t scratch_bytes, void* stream);
+
+/*
  * Sorted distinct elements of an array of `volume` elements (any shape: it is treated as
  * flat).  values_out must have room for `volume` elements; the number written goes to
  * *count_out (device memory, 8-byte aligned), which the caller reads after synchronising

@@ -114,3 +114,74 @@ def test_ties_specials_and_long_arrays(dtype, side):
         print(f"searchsorted dtype={np.dtype(dtype).name} n={n} side={side}", flush=True)
         got = np.asarray(num.searchsorted(a, v, side=side))
         assert np.array_equal(got, np.searchsorted(a, v, side=side)), (dtype, n, side)
+
+
+# ---- many queries into a large array: the library sorts the queries first (workspace entry
+# point) and stores every answer where its query came from ----
+
+def _reference_positions(a_sorted, v, side):
+    """numpy.searchsorted; for float16 / complex data with NaNs NumPy's own ordering of the
+    array and of the queries is the same one the library uses (NaN last, tiers for complex)."""
+    return np.searchsorted(a_sorted, v, side=side)
+
+
+@pytest.mark.parametrize("side", SIDES)
+@pytest.mark.parametrize("dtype", [np.int8, np.uint16, np.int32, np.float32, np.int64, np.float64,
+                                   np.complex64, np.complex128], ids=lambda d: np.dtype(d).name)
+def test_many_queries_large_array(dtype, side):
+    from cunumeric_amd import _lib
+    from cunumeric_amd.config import to_core_dtype
+
+    dt = np.dtype(dtype)
+    rng = np.random.default_rng(71)
+    n = (64 << 20) // dt.itemsize + 1001          # just past the size from which queries are sorted
+    m = (1 << 20) + 77
+    a = np.sort(random_array(dtype, n, rng, specials=True), kind="stable")
+    v = random_array(dtype, m, rng, specials=True)
+    v[: m // 8] = a[rng.integers(0, n, m // 8)]   # exact hits, so the two sides differ
+    assert _lib.load().misort_searchsorted_scratch_bytes(to_core_dtype(dt), n, m) > 0
+    print(f"searchsorted sorted queries dtype={dt.name} side={side}", flush=True)
+    got = np.asarray(num.searchsorted(num.array(a), num.array(v), side=side))
+    assert got.dtype == np.int64 and got.shape == v.shape
+    assert np.array_equal(got, _reference_positions(a, v, side))
+
+
+def test_workspace_entry_point_matches_the_plain_one():
+    """The same call with and without a workspace through the C ABI, 2-D queries."""
+    import torch
+
+    from cunumeric_amd import _lib
+    from cunumeric_amd.config import to_core_dtype
+
+    lib = _lib.load()
+    rng = np.random.default_rng(72)
+    n, m = (1 << 24) + 5, (1 << 20) + 3
+    a = np.sort(rng.standard_normal(n).astype(np.float32))
+    v = rng.standard_normal(m).astype(np.float32)
+    v[::7] = np.nan
+    v[1::7] = -0.0
+    dev = torch.device("cuda", 0)
+    d_a = torch.from_numpy(a.view(np.uint8)).to(dev)
+    d_v = torch.from_numpy(v.view(np.uint8)).to(dev)
+    code = to_core_dtype(np.dtype(np.float32))
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for with_ws in (False, True):
+        for left in (1, 0):
+            d_o = torch.full((m,), -1, dtype=torch.int64, device=dev)
+            need = lib.misort_searchsorted_scratch_bytes(code, n, m) if with_ws else 0
+            assert (need > 0) == with_ws
+            d_s = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+            _lib.check(lib.misort_searchsorted_ws(code, d_a.data_ptr(), n, d_v.data_ptr(), m, left,
+                                                  d_o.data_ptr(), d_s.data_ptr() if with_ws else None, need, stream))
+            torch.cuda.synchronize()
+            outs.append(d_o.cpu().numpy())
+    assert np.array_equal(outs[0], outs[2]) and np.array_equal(outs[1], outs[3])
+    assert np.array_equal(outs[0], np.searchsorted(a, v, side="left"))
+    assert np.array_equal(outs[1], np.searchsorted(a, v, side="right"))
+    # too small a workspace is refused before anything runs
+    d_o = torch.empty(m, dtype=torch.int64, device=dev)
+    d_s = torch.empty(4096, dtype=torch.uint8, device=dev)
+    rc = lib.misort_searchsorted_ws(code, d_a.data_ptr(), n, d_v.data_ptr(), m, 1, d_o.data_ptr(),
+                                    d_s.data_ptr(), 4096, stream)
+    assert rc == 4   # MISORT_ERR_SCRATCH
