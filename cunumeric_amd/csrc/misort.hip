@@ -51,6 +51,17 @@ static bool side_band_default()
   return v;
 }
 
+// Passes over a digit that is the same in every key are skipped unless the environment says
+// MISORT_SKIP_PASSES=0 when the library is first used.
+static bool skip_passes_default()
+{
+  static const bool v = [] {
+    const char* e = getenv("MISORT_SKIP_PASSES");
+    return !(e && *e == '0');
+  }();
+  return v;
+}
+
 static int fail(int code, const std::string& msg)
 {
   g_last_error = msg;
@@ -233,6 +244,10 @@ struct Plan {
   // byte carry, only where few digit values are in use; it says so per row in side_flag
   bool side_adaptive = false;
   size_t off_digits = 0, off_side_flag = 0;
+  // middle passes whose digit is the same in every key are skipped (decided on the device from
+  // the OR of the keys and of their complements, which the first upsweep leaves in key_bits)
+  bool skip_dead_passes = false;
+  size_t off_key_bits = 0;
   size_t off_gather_idx = 0, off_gather_src = 0;
   // counting sort of 2-byte keys: chunks of the histogram kernel, counters, their scan
   size_t c16_chunks = 0, c16_chunk_len = 0, off_c16_hist = 0, off_c16_prefix = 0;
@@ -348,6 +363,7 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.off_slab_tot      = take(pl.slab_tot_bytes);
     take(pl.slab_tot_bytes);
     pl.off_side_flag     = take(2 * pl.rows * sizeof(uint32_t));  // per pass parity and row
+    pl.off_key_bits      = take(KEY_BITS_SLOTS * 4 * sizeof(unsigned long long));
     pl.zero_bytes        = off - pl.off_special_ctr;
     pl.off_chunk_hist    = take(pl.n_chunks * RADIX * sizeof(uint32_t));
 
@@ -365,6 +381,9 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     }
     // (8-byte keys: the upsweep saves 7 of 8 bytes per key; with 4-byte keys the extra
     // stores of the scatter cost more than the upsweep saves)
+    // (not for keys-only float sorts: the patch of their zeros and NaNs counts on which of the
+    // two buffers the last pass leaves free)
+    pl.skip_dead_passes = skip_passes_default() && pl.n_passes >= 3 && !pl.specials;
     pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
     pl.side_adaptive = side_band_default() && !pl.side_band && pl.n_passes >= 2 && pl.dt.bytes >= 4 &&
                        (pl.pay != PAY_NONE || pl.dt.bytes > 4);
@@ -472,7 +491,7 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
   const dim3 grid((unsigned)pl.n_chunks);
 
   L.run(K_UPSWEEP, [&] {
-    if (pp.digits_in && !pp.side_flag_in) {  // the pass before always writes the side-band
+    if (pp.digits_in && !pp.side_flags) {  // the last live pass always writes the side-band
       hipLaunchKernelGGL((upsweep_digits_kernel<kUpsweepDigitThreads>), grid, dim3(kUpsweepDigitThreads), 0,
                          L.stream, pp);
       return;
@@ -544,6 +563,11 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
   pp.xform           = pl.dt.xform;
   pp.rank_by_add     = rank_by_add_default();
+  pp.n_rows          = (uint32_t)pl.rows;
+  pp.key_buf[0]      = S + pl.off_keys[0];
+  pp.key_buf[1]      = S + pl.off_keys[1];
+  pp.pay_buf[0]      = PAY != PAY_NONE ? S + pl.off_pay[0] : nullptr;
+  pp.pay_buf[1]      = PAY != PAY_NONE ? S + pl.off_pay[1] : nullptr;
 
   const void* cur_keys = vin;
   const void* cur_pay  = iin;
@@ -580,9 +604,14 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
       uint8_t* side = (pl.side_band || pl.side_adaptive) ? reinterpret_cast<uint8_t*>(S + pl.off_digits) : nullptr;
       pp.digits_in  = first ? nullptr : side;  // written by the pass before
       pp.digits_out = last ? nullptr : side;   // read by the next upsweep, which runs after this scatter
-      uint32_t* flag   = reinterpret_cast<uint32_t*>(S + pl.off_side_flag);
-      pp.side_flag_in  = (pl.side_adaptive && !first) ? flag + ((pass - 1) & 1) * pl.rows : nullptr;
-      pp.side_flag_out = (pl.side_adaptive && !last) ? flag + (pass & 1) * pl.rows : nullptr;
+      pp.side_flags = pl.side_adaptive ? reinterpret_cast<uint32_t*>(S + pl.off_side_flag) : nullptr;
+    }
+    pp.pass     = pass;
+    pp.n_passes = pl.n_passes;
+    {
+      unsigned long long* bits = reinterpret_cast<unsigned long long*>(S + pl.off_key_bits);
+      pp.key_bits_out = (pl.skip_dead_passes && first) ? bits : nullptr;
+      pp.key_bits     = pl.skip_dead_passes ? bits : nullptr;  // complete once the first upsweep has run
     }
     pp.slab_tot = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + (pass & 1) * pl.slab_tot_bytes);
     pp.slab_tot_next =
@@ -1112,6 +1141,10 @@ int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int arg
            sname[pl.strategy], pl.dt.bytes, pl.n_passes, RADIX_BITS, pl.tile, pl.rows, pl.row_len,
            pl.chunks_per_row, pl.tiles_per_chunk, pname[pl.pay], (int)pl.specials,
            (int)pl.gather_values, pl.side_band ? 1 : (pl.side_adaptive ? 2 : 0), pl.total);
+  if (pl.skip_dead_passes) {
+    const size_t len = strlen(buf);
+    if (len + 16 < buf_bytes) snprintf(buf + len, buf_bytes - len, " skip_dead_passes=1");
+  }
   return MISORT_OK;
 }
 

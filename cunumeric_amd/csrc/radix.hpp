@@ -71,8 +71,22 @@ struct PassParams {
   const uint8_t* digits_in;  // this pass's digit of every key of keys_in, or NULL (upsweep_digits_kernel)
   uint8_t* digits_out;       // downsweep: the NEXT pass's digit of every key written (always with
                              // SIDE, otherwise only where the pass decides that it pays), or NULL
-  const uint32_t* side_flag_in;  // [rows] 1 where the pass before wrote digits_in for the row, or NULL
-  uint32_t* side_flag_out;       // [rows] where this pass says whether it writes digits_out, or NULL
+  uint32_t* side_flags;      // [2][n_rows], or NULL: entry [k & 1][row] = 1 where pass k wrote digits_out
+                             // for the row (passes that decide it per row)
+  uint32_t n_rows;
+  int pass, n_passes;        // which pass this is, of how many
+  // Passes whose digit is the same in every key move nothing and are skipped, decided on the
+  // device: the first upsweep ORs all keys and all complemented keys into key_bits_out
+  // (KEY_BITS_SLOTS copies of {or lo, or hi, or-of-complement lo, hi}); a bit varies iff it
+  // is set in both.  Every later
+  // kernel reads the four words (key_bits) and works out for itself which middle passes are
+  // dead, hence which of the two ping-pong buffers holds its input (key_buf / pay_buf; the
+  // keys_in .. pay_out above are what they would be with no pass skipped), and which pass is
+  // the next live one (whose digit the side-band carries).  NULL: no pass is skipped.
+  const unsigned long long* key_bits;
+  unsigned long long* key_bits_out;
+  void* key_buf[2];
+  void* pay_buf[2];
   const void* pay_in;    // PAY_IDX32: u32 (ignored when FIRST); PAY_I64: int64, NULL => positions
   void* pay_out;         // PAY_IDX32: u32, int64 when LAST; PAY_I64: int64
   uint32_t* chunk_hist;             // [rows * chunks_per_row][RADIX] counts of this pass
@@ -94,6 +108,55 @@ struct PassParams {
   int rank_by_add;    // downsweep: rank with returning LDS adds where the chunk's digits allow
   const void* pivot;  // PART passes: one pivot key per row
 };
+
+// key_bits holds this many copies of its four words (their OR counts)
+constexpr int KEY_BITS_SLOTS = 8;
+
+// What a kernel of pass p.pass works out from key_bits (all of it uniform).
+struct PassPlan {
+  bool skip;        // this pass moves nothing
+  uint32_t parity;  // dead passes before this one, modulo 2: the ping-pong buffers are swapped
+  int next_shift;   // digit position of the next live pass
+  int prev_live;    // the last live pass before this one
+};
+__device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
+{
+  PassPlan r{false, 0u, p.shift + RADIX_BITS, p.pass - 1};
+  if (!p.key_bits) return r;
+  auto uniform64 = [](unsigned long long v) {  // same in every lane: keep it in scalar registers
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return ((unsigned long long)b << 32) | a;
+  };
+  unsigned long long w[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int sl = 0; sl < KEY_BITS_SLOTS; ++sl) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] |= p.key_bits[4 * sl + i];
+  }
+  const unsigned long long lo = uniform64(w[0] & w[2]);
+  const unsigned long long hi = uniform64(w[1] & w[3]);
+  auto dead = [&](int j) {  // first and last pass transform the elements: never skipped
+    if (j <= 0 || j >= p.n_passes - 1) return false;
+    const unsigned long long w = j < 8 ? lo : hi;
+    return ((w >> (8 * (j & 7))) & 0xFFull) == 0;
+  };
+  for (int j = 1; j < p.pass; ++j) r.parity ^= dead(j) ? 1u : 0u;
+  r.skip = dead(p.pass);
+  int nx = p.pass + 1;
+  while (dead(nx)) ++nx;
+  r.next_shift = nx * RADIX_BITS;
+  int pv = p.pass - 1;
+  while (dead(pv)) --pv;
+  r.prev_live = pv;
+  return r;
+}
+// index of the ping-pong buffer that holds the input of pass p.pass (>= 1)
+__device__ __forceinline__ uint32_t input_buffer(const PassParams& p, const PassPlan& pl)
+{
+  return (uint32_t)((p.pass - 1) & 1) ^ pl.parity;
+}
+
 
 template <typename T>
 __device__ __forceinline__ T wave_incl_scan(T v, int lane)
@@ -151,11 +214,9 @@ __device__ __forceinline__ void lds_barrier()
 // never queue on a bank.
 // ---------------------------------------------------------------------------------------
 template <int NT>
-__device__ __forceinline__ void count_digit_bytes(const PassParams& p, uint32_t* h /* LDS, RADIX * 32 words */)
+__device__ __forceinline__ void count_digit_bytes(const PassParams& p, uint32_t* h /* LDS, RADIX * 32 words, zeroed */)
 {
   constexpr int COPIES = 32;
-  for (int i = threadIdx.x; i < RADIX * COPIES; i += NT) h[i] = 0;
-  __syncthreads();
   const uint32_t row   = blockIdx.x / p.chunks_per_row;
   const uint32_t chunk = blockIdx.x % p.chunks_per_row;
   const uint64_t clen  = (uint64_t)p.tiles_per_chunk * p.tile;
@@ -200,6 +261,10 @@ template <int NT>
 __global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
 {
   __shared__ __attribute__((aligned(16))) uint32_t h[RADIX * 32];
+  for (int i = threadIdx.x; i < RADIX * 32; i += NT) h[i] = 0;  // (while the plan's words arrive)
+  const bool skip = plan_pass(p).skip;
+  __syncthreads();
+  if (skip) return;
   count_digit_bytes<NT>(p, h);
 }
 
@@ -218,16 +283,24 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   constexpr int COPIES = 4;
   constexpr int WORDS  = NW * RADIX * COPIES > RADIX * 32 ? NW * RADIX * COPIES : RADIX * 32;
   __shared__ __attribute__((aligned(16))) uint32_t lhist[WORDS];
+  __shared__ unsigned long long wg_bits[FIRST ? NW * 4 : 1];
   const uint32_t row   = blockIdx.x / p.chunks_per_row;
   const uint32_t chunk = blockIdx.x % p.chunks_per_row;
-  if constexpr (!FIRST && !SPECIALS && !PART) {
-    // the pass before wrote this pass's digits as bytes for this row: count those
-    if (p.side_flag_in && p.side_flag_in[row]) {
-      count_digit_bytes<NT>(p, lhist);
-      return;
+  // (the counters are cleared while the words of the plan arrive)
+  for (int i = threadIdx.x; i < ((!FIRST && !PART && !SPECIALS) ? WORDS : NW * RADIX * COPIES); i += NT) lhist[i] = 0;
+  if constexpr (!FIRST && !PART) {
+    const PassPlan plan = plan_pass(p);
+    if (plan.skip) return;  // every key has the same digit: the scatter of this pass is skipped too
+    if (p.key_bits) p.keys_in = input_buffer(p, plan) ? p.key_buf[1] : p.key_buf[0];
+    if constexpr (!SPECIALS) {
+      // the last live pass wrote this pass's digits as bytes for this row: count those
+      if (p.digits_in && p.side_flags && p.side_flags[(uint64_t)(plan.prev_live & 1) * p.n_rows + row]) {
+        __syncthreads();
+        count_digit_bytes<NT>(p, lhist);
+        return;
+      }
     }
   }
-  for (int i = threadIdx.x; i < NW * RADIX * COPIES; i += NT) lhist[i] = 0;
   __syncthreads();
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -248,8 +321,21 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   if constexpr (PART) pivot = reinterpret_cast<const KeyT*>(p.pivot)[row];
 
   uint32_t n_zero = 0, n_nan = 0, n_negzero = 0, n_neg = 0;
+  // FIRST: OR of the keys and of their complements (which bits vary over the whole input)
+  unsigned long long or_lo = 0, or_hi = 0, nor_lo = 0, nor_hi = 0;
   auto count = [&](KeyT raw) {
     const KeyT k = FIRST ? KeyOps<KeyT>::to_key(raw, p.xform) : raw;
+    if constexpr (FIRST && !PART) {
+      if constexpr (sizeof(KeyT) == 16) {
+        or_lo |= k.lo;
+        or_hi |= k.hi;
+        nor_lo |= ~k.lo;
+        nor_hi |= ~k.hi;
+      } else {
+        or_lo |= (unsigned long long)k;
+        nor_lo |= (unsigned long long)(KeyT)~k;
+      }
+    }
     atomicAdd(&my[pass_digit<KeyT, PART>(k, p.shift, pivot) * COPIES], 1u);
     if constexpr (SPECIALS) {
       using F = FloatBits<KeyT>;
@@ -303,7 +389,36 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       if (n_neg) atomicAdd(&ctr[3], (unsigned long long)n_neg);
     }
   }
+  if constexpr (FIRST && !PART) {
+    if (p.key_bits_out) {
+#pragma unroll
+      for (int s = 32; s > 0; s >>= 1) {
+        or_lo |= __shfl_xor(or_lo, s, 64);
+        nor_lo |= __shfl_xor(nor_lo, s, 64);
+        if (sizeof(KeyT) == 16) {
+          or_hi |= __shfl_xor(or_hi, s, 64);
+          nor_hi |= __shfl_xor(nor_hi, s, 64);
+        }
+      }
+      if (lane == 0) {
+        wg_bits[wave * 4 + 0] = or_lo;
+        wg_bits[wave * 4 + 1] = or_hi;
+        wg_bits[wave * 4 + 2] = nor_lo;
+        wg_bits[wave * 4 + 3] = nor_hi;
+      }
+    }
+  }
   __syncthreads();
+  if constexpr (FIRST && !PART) {
+    // Atomics on one address queue up (about 10 ns each), so a workgroup adds its bits once,
+    // to one of KEY_BITS_SLOTS copies of the words, and nobody waits for the result.
+    if (p.key_bits_out && threadIdx.x < 4 && (sizeof(KeyT) == 16 || (threadIdx.x & 1) == 0)) {
+      unsigned long long v = 0;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v |= wg_bits[w * 4 + threadIdx.x];
+      atomicOr(&p.key_bits_out[4 * (blockIdx.x % KEY_BITS_SLOTS) + threadIdx.x], v);
+    }
+  }
   uint32_t* out = p.chunk_hist + (uint64_t)blockIdx.x * RADIX;
   unsigned long long* slab =
     p.slab_tot + ((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX;
@@ -419,6 +534,30 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   KeyT pivot{};
   if constexpr (PART) pivot = reinterpret_cast<const KeyT*>(p.pivot)[row];
   auto digit_of = [&](KeyT k) { return pass_digit<KeyT, PART>(k, p.shift, pivot); };
+  int next_shift = p.shift + RADIX_BITS;  // digit position that the side-band carries
+  if constexpr (!PART && sizeof(KeyT) >= 4) {  // (shorter keys have no middle pass)
+    const PassPlan plan = plan_pass(p);
+    if (plan.skip) {
+      // Every key of the input has the same digit here: the pass would copy every row onto
+      // itself, so it moves nothing and the data stays in the buffer it is in (later kernels
+      // work that out the same way).  What it owes the next pass remains: zeroed slab totals.
+      if (p.slab_tot_next && chunk < p.slabs_per_row && tid < RADIX)
+        p.slab_tot_next[((uint64_t)row * p.slabs_per_row + chunk) * RADIX + tid] = 0;
+      return;
+    }
+    next_shift = plan.next_shift;
+    if (p.key_bits) {
+      const bool cur = input_buffer(p, plan) != 0;
+      if (!FIRST) {
+        p.keys_in = cur ? p.key_buf[1] : p.key_buf[0];
+        p.pay_in  = cur ? p.pay_buf[1] : p.pay_buf[0];
+      }
+      if (!LAST) {
+        p.keys_out = cur ? p.key_buf[0] : p.key_buf[1];
+        p.pay_out  = cur ? p.pay_buf[0] : p.pay_buf[1];
+      }
+    }
+  }
 
   // thread d < RADIX owns digit value d: global position of its next unwritten element
   // and how many elements of it wait in the carry
@@ -444,7 +583,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
     } else {
       kout[dst] = k;
       if constexpr (ADAPT) {
-        if (side_on) p.digits_out[dst] = (uint8_t)KeyOps<KeyT>::digit(k, p.shift + RADIX_BITS);
+        if (side_on) p.digits_out[dst] = (uint8_t)KeyOps<KeyT>::digit(k, next_shift);
       }
     }
     if (PAY == PAY_IDX32) {
@@ -543,7 +682,8 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
     if constexpr (ADAPT) {
       if (p.digits_out) {
         side_on = __builtin_amdgcn_readfirstlane((int)(present <= kSidePresentMax * 65536u)) != 0;
-        if (chunk == 0 && tid == 0 && p.side_flag_out) p.side_flag_out[row] = side_on ? 1u : 0u;
+        if (chunk == 0 && tid == 0 && p.side_flags)
+          p.side_flags[(uint64_t)(p.pass & 1) * p.n_rows + row] = side_on ? 1u : 0u;
       }
     }
     if (tid < RADIX) run = row_base + base + incl - total + before;
@@ -653,7 +793,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
             emit(orun[j] + e, bk[j], PAY == PAY_NONE ? PayT{} : bv[PAY == PAY_NONE ? 0 : j]);
             if constexpr (SIDE) {
               const int32_t eb = (int32_t)((tb[j] >> 16) & 0xFFu) - 128;
-              const uint32_t b = KeyOps<KeyT>::digit(bk[j], p.shift + RADIX_BITS);
+              const uint32_t b = KeyOps<KeyT>::digit(bk[j], next_shift);
               if ((int32_t)e < eb) {
                 p.digits_out[orun[j] + e] = (uint8_t)b;
               } else {
@@ -707,7 +847,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
             emit(abase[i] + q, ak[i], v);
             if constexpr (SIDE) {
               const int32_t blim = lim - (alim[i] & 0xFF);
-              const uint32_t b   = KeyOps<KeyT>::digit(ak[i], p.shift + RADIX_BITS);
+              const uint32_t b   = KeyOps<KeyT>::digit(ak[i], next_shift);
               if ((int32_t)q < blim)
                 p.digits_out[abase[i] + q] = (uint8_t)b;
               else

@@ -1,0 +1,109 @@
+"""Radix passes over a digit that is the same in every key are skipped on the device (the
+first upsweep ORs the keys and their complements; every later kernel derives from those
+words which middle passes are dead and which ping-pong buffer holds its input).  Inputs whose
+constant bytes sit in every combination of positions, for all key widths with middle passes,
+sorts and argsorts, rows, a caller payload, and the same input with the skipping switched
+off must agree with NumPy."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from tests.util import Abi, bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def abi():
+    return Abi()
+
+
+def masked_random(dtype, n, rng, live_bytes):
+    """Unsigned random values in which only the bytes listed in live_bytes vary; the others
+    carry a fixed non-zero pattern."""
+    dt = np.dtype(dtype)
+    u = np.dtype(f"u{dt.itemsize}")
+    x = rng.integers(0, np.iinfo(u).max, n, dtype=u, endpoint=True)
+    mask = sum(0xFF << (8 * b) for b in live_bytes)
+    const = rng.integers(0, np.iinfo(u).max, dtype=u, endpoint=True)
+    x = (x & u.type(mask)) | (const & u.type(~mask & np.iinfo(u).max))
+    return x.view(dt) if dt.kind != "u" else x
+
+
+WIDTH4 = [(0,), (0, 1), (0, 3), (1, 2), (3,), (0, 1, 2, 3), (), (2,)]
+WIDTH8 = [(0,), (0, 1), (0, 7), (3, 4), (7,), (1, 2, 3, 4, 5, 6), (0, 2, 4, 6), (), (0, 1, 2, 3, 4, 5, 6, 7), (5,)]
+
+
+@pytest.mark.parametrize("dtype,patterns", [(np.uint32, WIDTH4), (np.int32, WIDTH4), (np.uint64, WIDTH8),
+                                             (np.int64, WIDTH8)], ids=["uint32", "int32", "uint64", "int64"])
+def test_constant_bytes_in_every_position(abi, dtype, patterns):
+    rng = np.random.default_rng(61)
+    n = 300007
+    for live in patterns:
+        a = masked_random(dtype, n, rng, live)
+        for chunks in (0, 3):
+            print(f"skip passes dtype={np.dtype(dtype).name} live bytes={live} chunks={chunks}", flush=True)
+            assert np.array_equal(abi.local_sort(a, n, argsort=False, chunks=chunks), np.sort(a, kind="stable")), live
+            assert np.array_equal(abi.local_sort(a, n, argsort=True, chunks=chunks), np.argsort(a, kind="stable")), live
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32, np.float64, np.complex64, np.complex128],
+                         ids=lambda d: np.dtype(d).name)
+def test_small_ranges_rows_and_payload(abi, dtype):
+    """Values from a small range (the usual case for integer data): the upper digits of the
+    keys are constant.  Floats and complex numbers built from small integers have constant
+    low mantissa bytes instead."""
+    rng = np.random.default_rng(62)
+    rows, row_len = 3, 120001
+    a = rng.integers(0, 1000, rows * row_len).astype(dtype).reshape(rows, row_len)
+    if np.dtype(dtype).kind == "c":
+        a = a + 1j * rng.integers(0, 50, a.shape).astype(a.real.dtype)
+    print(f"skip passes small range dtype={np.dtype(dtype).name}", flush=True)
+    got = abi.local_sort(a, row_len, argsort=True, chunks=2 * rows).reshape(rows, row_len)
+    assert np.array_equal(got, np.argsort(a, axis=1, kind="stable"))
+    got = abi.local_sort(a, row_len, argsort=False).reshape(rows, row_len)
+    assert bits_equal(got, np.sort(a, axis=1, kind="stable"))
+    pay = rng.integers(-(2**62), 2**62, rows * row_len, dtype=np.int64)
+    got = abi.local_sort(a, row_len, argsort=True, indices_in=pay).reshape(rows, row_len)
+    ref = np.take_along_axis(pay.reshape(rows, row_len), np.argsort(a, axis=1, kind="stable"), axis=1)
+    assert np.array_equal(got, ref)
+    # in place
+    flat = a.reshape(-1).copy()
+    got = abi.local_sort(flat[:row_len], row_len, argsort=False, inplace=True)
+    assert bits_equal(got, np.sort(flat[:row_len], kind="stable"))
+
+
+def test_large_int64_small_range(abi):
+    rng = np.random.default_rng(63)
+    n = 1 << 24
+    a = rng.integers(0, 50000, n, dtype=np.int64)
+    print("skip passes int64 2^24 values below 50000", flush=True)
+    assert np.array_equal(abi.local_sort(a, n, argsort=True), np.argsort(a, kind="stable"))
+    assert np.array_equal(abi.local_sort(a, n, argsort=False), np.sort(a))
+    assert "skip_dead_passes=1" in abi.describe_plan(np.int64, n, n, True)
+
+
+def test_switch_off_gives_the_same_result():
+    code = (
+        "import numpy as np, sys\n"
+        "from tests.util import Abi\n"
+        "rng = np.random.default_rng(64)\n"
+        "a = rng.integers(0, 300, 400001, dtype=np.int64)\n"
+        "abi = Abi()\n"
+        "plan = abi.describe_plan(np.int64, a.size, a.size, True)\n"
+        "s = abi.local_sort(a, a.size, argsort=True, chunks=3)\n"
+        "sys.stdout.write(plan + '\\n' + str(bool((s == np.argsort(a, kind='stable')).all())) + '\\n')\n"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    outs = []
+    for flag in ("1", "0"):
+        env = dict(os.environ, MISORT_SKIP_PASSES=flag, PYTHONPATH=root)
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, cwd=root,
+                           timeout=240)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs.append(r.stdout.strip().splitlines())
+    assert outs[0][-1] == "True" and outs[1][-1] == "True"
+    assert "skip_dead_passes=1" in outs[0][0] and "skip_dead_passes" not in outs[1][0]
