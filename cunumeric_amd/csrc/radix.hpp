@@ -10,6 +10,9 @@
 //                     the digit values and over the chunks before its own (where its keys of
 //                     each digit value start), then it walks its tiles in order, carrying the
 //                     running start of every digit value, so no workgroup ever waits on another.
+// Middle passes whose digit is the same in every key are skipped: the first upsweep ORs the
+// keys and their complements, every later kernel works out the rest from those words
+// (plan_pass).
 // Keys-only sorts of 8-byte elements: every pass but the last also writes the next pass's digit
 // of each key as a byte (SIDE), which the next upsweep counts instead of the keys
 // (upsweep_digits_kernel).
