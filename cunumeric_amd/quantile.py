@@ -1,7 +1,11 @@
-"""``quantile`` / ``percentile``: the callers of the sort path in the reference's statistics
-section (cunumeric/module.py:8339-8531 ``quantile``, 8534-8644 ``percentile``, which sort the
-array along the reduction axis with ``sort`` / ``ndarray.sort`` at :8472-8476 and then read
-the two order statistics around each quantile, ``quantile_impl`` :8248-8336).
+"""``quantile`` / ``percentile`` / ``nanquantile`` / ``nanpercentile``: the callers of the sort
+path in the reference's statistics section (cunumeric/module.py:8339-8531 ``quantile``,
+8534-8644 ``percentile``, which sort the array along the reduction axis with ``sort`` /
+``ndarray.sort`` at :8472-8476 and then read the two order statistics around each quantile,
+``quantile_impl`` :8248-8336; :8757-8962 ``nanquantile`` and :8965-9065 ``nanpercentile``, which
+count the non-NaN elements of every slice, sort with the NaNs moved behind everything else
+(:8901-8903) and read the order statistics of each slice's own length, ``nanquantile_impl``
+:8647-8754).
 
 Same arguments, result shapes / dtypes and exceptions.  The order statistics come from the
 GPU sort of this package; for ONE quantile over a flat array or long rows they come from the
@@ -139,25 +143,11 @@ def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool) 
     return {k: t[..., k] for k in wanted}
 
 
-def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: Optional[ndarray] = None,
-             overwrite_input: bool = False, method: str = "linear", keepdims: bool = False) -> ndarray:
-    """The q-th quantile(s) of ``a`` along ``axis`` (``None``: of the flattened array; several
-    axes: of their product).  Result shape: ``q.shape`` followed by the shape of ``a`` without
-    the reduced axes (kept with extent 1 under ``keepdims``); dtype: the input's for the methods
-    that return a sample, float64 otherwise; complex input is a TypeError, a wrongly shaped
-    ``out`` a ValueError (reference: cunumeric/module.py:8339-8531)."""
-    if method not in METHODS:
-        raise ValueError(f"{method!r} is not a valid method. Use one of: {', '.join(METHODS)}")
-    a = convert_to_cunumeric_ndarray(a)
-    if a.dtype.kind == "c":
-        raise TypeError("input array cannot be of complex type")
-    q_arr = np.asarray(q, dtype=np.float64)
-    if q_arr.size and not (np.all(q_arr >= 0) and np.all(q_arr <= 1)):
-        raise ValueError("Quantiles must be in the range [0, 1]")
+def _reduction_rows(a: ndarray, axis):
+    """``a`` with the reduction axes moved last and merged into one: (rows, axes, shape of the
+    kept axes, original shape, whether that needed a copy)."""
     original_shape = a.shape
     nd = a.ndim
-
-    # ---- the reduction axes last, merged into one --------------------------------------
     if axis is None:
         axes = tuple(range(nd))
     elif isinstance(axis, Iterable):
@@ -184,12 +174,30 @@ def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: 
     if nd and (kept + axes) != tuple(range(nd)):
         # a dense copy with the reduced axes moved behind the others (never sorted in place)
         moved = a.to_torch().permute(*kept, *axes).contiguous()
-        rows = _from_torch(moved.reshape(*kept_shape, n), a.dtype)
-        overwrite_input = False
-    else:
-        rows = a.reshape((*kept_shape, n))
-        if len(axes) > 1 and axis is not None:
-            overwrite_input = False  # as the reference: only a single axis is sorted in place
+        return _from_torch(moved.reshape(*kept_shape, n), a.dtype), axes, kept_shape, original_shape, True
+    return a.reshape((*kept_shape, n)), axes, kept_shape, original_shape, False
+
+
+def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: Optional[ndarray] = None,
+             overwrite_input: bool = False, method: str = "linear", keepdims: bool = False) -> ndarray:
+    """The q-th quantile(s) of ``a`` along ``axis`` (``None``: of the flattened array; several
+    axes: of their product).  Result shape: ``q.shape`` followed by the shape of ``a`` without
+    the reduced axes (kept with extent 1 under ``keepdims``); dtype: the input's for the methods
+    that return a sample, float64 otherwise; complex input is a TypeError, a wrongly shaped
+    ``out`` a ValueError (reference: cunumeric/module.py:8339-8531)."""
+    if method not in METHODS:
+        raise ValueError(f"{method!r} is not a valid method. Use one of: {', '.join(METHODS)}")
+    a = convert_to_cunumeric_ndarray(a)
+    if a.dtype.kind == "c":
+        raise TypeError("input array cannot be of complex type")
+    q_arr = np.asarray(q, dtype=np.float64)
+    if q_arr.size and not (np.all(q_arr >= 0) and np.all(q_arr <= 1)):
+        raise ValueError("Quantiles must be in the range [0, 1]")
+    rows, axes, kept_shape, original_shape, moved = _reduction_rows(a, axis)
+    nd = a.ndim
+    n = rows.shape[-1]
+    if moved or (len(axes) > 1 and axis is not None):
+        overwrite_input = False  # as the reference: only a single axis is sorted in place
 
     # ---- the samples around every quantile ---------------------------------------------
     places = [_position(method, float(qv), n) for qv in q_arr.reshape(-1)]
@@ -238,3 +246,118 @@ def percentile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out
         raise ValueError("Percentiles must be in the range [0, 100]")
     return quantile(a, q_arr, axis=axis, out=out, overwrite_input=overwrite_input, method=method,
                     keepdims=keepdims)
+
+
+def _position_rows(method: str, q: float, n: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``_position`` for samples of different sizes at once: ``n`` holds the size of every
+    sample (int64, >= 1); returns int64 lo, hi and float64 g of the same shape."""
+    nf = n.to(torch.float64)
+    last = nf - 1.0
+
+    def clipped(v, weight):
+        lo = torch.floor(v)
+        g = weight(v - lo, v)
+        over, under = v >= last, v < 0
+        lo_c = torch.where(over, last, torch.where(under, torch.zeros_like(v), lo))
+        hi_c = torch.where(over | under, lo_c, lo + 1.0)
+        g_c = torch.where(over | under, torch.zeros_like(v), g)
+        return lo_c.to(torch.int64), hi_c.to(torch.int64), g_c
+
+    if method in _CONTINUOUS or method == "linear":
+        if method == "linear":
+            v = last * q
+        else:
+            alpha, beta = _CONTINUOUS[method]
+            v = nf * q + (alpha + q * (1.0 - alpha - beta)) - 1.0
+        return clipped(v, lambda frac, _: frac)
+    if method == "averaged_inverted_cdf":
+        return clipped(nf * q - 1.0, lambda frac, _: torch.where(frac == 0, 0.5, 1.0).to(torch.float64))
+    if method == "midpoint":
+        v = 0.5 * (torch.floor(last * q) + torch.ceil(last * q))
+        return clipped(v, lambda frac, _: torch.where(frac == 0, 0.0, 0.5).to(torch.float64))
+    if method == "inverted_cdf":
+        v = nf * q - 1.0
+        lo = torch.floor(v)
+        i = torch.where(v == lo, lo, lo + 1.0)
+    elif method == "closest_observation":
+        v = nf * q - 1.5
+        lo = torch.floor(v)
+        odd = torch.remainder(lo, 2.0) == 1.0
+        i = torch.where((v == lo) & odd, lo, lo + 1.0)
+    elif method == "lower":
+        i = torch.floor(last * q)
+    elif method == "higher":
+        i = torch.ceil(last * q)
+    elif method == "nearest":
+        i = torch.round(last * q)  # half to even
+    else:
+        raise ValueError(f"{method!r} is not a valid method. Use one of: {', '.join(METHODS)}")
+    i = torch.minimum(torch.clamp(i, min=0.0), last).to(torch.int64)
+    return i, i, torch.zeros_like(nf)
+
+
+def nanquantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: Optional[ndarray] = None,
+                overwrite_input: bool = False, method: str = "linear", keepdims: bool = False) -> ndarray:
+    """The q-th quantile(s) of ``a`` along ``axis``, ignoring NaNs: every slice is its non-NaN
+    elements (the sort of this package puts NaNs last, so they are the tail of the sorted
+    slice); a slice of NaNs only gives NaN.  Shapes, dtypes and exceptions as ``quantile``
+    (reference: cunumeric/module.py:8757-8962, 8647-8754)."""
+    from .module import sort
+
+    if method not in METHODS:
+        raise ValueError(f"{method!r} is not a valid method. Use one of: {', '.join(METHODS)}")
+    a = convert_to_cunumeric_ndarray(a)
+    if a.dtype.kind == "c":
+        raise TypeError("input array cannot be of complex type")
+    q_arr = np.asarray(q, dtype=np.float64)
+    if q_arr.size and not (np.all(q_arr >= 0) and np.all(q_arr <= 1)):
+        raise ValueError("Quantiles must be in the range [0, 1]")
+    rows, axes, kept_shape, original_shape, _ = _reduction_rows(a, axis)
+    nd = a.ndim
+    t = sort(rows, axis=-1).to_torch()
+    if a.dtype.kind == "f":
+        count = (~torch.isnan(t)).sum(dim=-1)
+    else:
+        count = torch.full(kept_shape, t.shape[-1], dtype=torch.int64, device=t.device)
+    empty = count == 0
+    n = torch.clamp(count, min=1)
+    to_dtype = a.dtype if method in _SAMPLE_METHODS else np.dtype(np.float64)
+    tdt = _torch_dtype(to_dtype)
+    results = []
+    for qv in q_arr.reshape(-1):
+        lo, hi, g = _position_rows(method, float(qv), n)
+        x = t.gather(-1, lo.unsqueeze(-1)).squeeze(-1).to(tdt)
+        if method in _SAMPLE_METHODS:
+            r = x
+        else:
+            y = t.gather(-1, hi.unsqueeze(-1)).squeeze(-1).to(tdt)
+            d = y - x
+            # the upper sample anchors the blend from the middle on, as in NumPy
+            r = torch.where(g == 0, x, torch.where(g < 0.5, x + d * g, y - d * (1.0 - g)))
+        if a.dtype.kind == "f":
+            r = torch.where(empty, torch.tensor(float("nan"), dtype=tdt, device=r.device), r)
+        results.append(r)
+    res = torch.stack(results, dim=0) if results else torch.empty((0, *kept_shape), dtype=tdt, device=t.device)
+    if keepdims:
+        remaining = tuple(1 if k in axes else original_shape[k] for k in range(nd))
+    else:
+        remaining = kept_shape
+    shape = (*q_arr.shape, *remaining)
+    res = res.reshape(shape)
+    if out is not None:
+        if tuple(out.shape) != shape:
+            raise ValueError("wrong shape on output array")
+        out.to_torch().copy_(res.to(_torch_dtype(out.dtype)))
+        return out
+    return _from_torch(res, to_dtype)
+
+
+def nanpercentile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: Optional[ndarray] = None,
+                  overwrite_input: bool = False, method: str = "linear", keepdims: bool = False) -> ndarray:
+    """The q-th percentile(s), ignoring NaNs: ``nanquantile`` with ``q / 100``
+    (reference: cunumeric/module.py:8965-9065)."""
+    q_arr = np.true_divide(np.asarray(q, dtype=np.float64), 100.0)
+    if q_arr.size and not (np.all(q_arr >= 0) and np.all(q_arr <= 1)):
+        raise ValueError("Percentiles must be in the range [0, 100]")
+    return nanquantile(a, q_arr, axis=axis, out=out, overwrite_input=overwrite_input, method=method,
+                       keepdims=keepdims)

@@ -31,3 +31,22 @@ def test_position_matches_numpy(method):
 def test_unknown_method():
     with pytest.raises(ValueError):
         _position("median", 0.5, 10)
+
+
+@pytest.mark.parametrize("method", METHODS)
+def test_positions_of_many_sample_sizes_at_once(method):
+    """The tensor form used by nanquantile (every slice has its own number of non-NaN
+    elements) names the same two samples and weight as the scalar form."""
+    import torch
+
+    from cunumeric_amd.quantile import _position_rows
+
+    sizes = list(range(1, 70)) + [100, 101, 1000, 4097]
+    n = torch.tensor(sizes, dtype=torch.int64)
+    for q in [0.0, 1.0, 0.5, 0.25, 0.75, 1 / 3, 2 / 3, 0.001, 0.999, 0.37, 0.42, 0.67, 0.83, 0.99, 0.39, 0.49,
+              0.1, 0.2, 0.3, 0.6]:
+        lo, hi, g = _position_rows(method, q, n)
+        for k, size in enumerate(sizes):
+            a, b, w = _position(method, q, size)
+            assert (int(lo[k]), int(hi[k])) == (a, b) or (w == 0.0 and float(g[k]) == 0.0 and int(lo[k]) == a), (q, size)
+            assert float(g[k]) == pytest.approx(w, abs=1e-12), (q, size)
