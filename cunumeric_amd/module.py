@@ -9,6 +9,7 @@ from __future__ import annotations
 from typing import Any, Optional, Sequence, Union
 
 import numpy as np
+import torch
 
 from .array import convert_to_cunumeric_ndarray, ndarray
 
@@ -40,6 +41,33 @@ def searchsorted(a: Any, v: Any, side: str = "left", sorter: Optional[Any] = Non
     """Indices into the sorted 1-D array ``a`` at which the elements of ``v`` would be
     inserted to keep it sorted (reference: cunumeric/module.py:6959-6996)."""
     return convert_to_cunumeric_ndarray(a).searchsorted(v, side, sorter)
+
+
+def digitize(x: Any, bins: Any, right: bool = False) -> ndarray:
+    """Index of the bin every element of ``x`` belongs to: ``searchsorted`` of ``x`` into the
+    monotonic 1-D ``bins`` with the side swapped; decreasing bins are searched reversed and the
+    result counted from the other end.  Complex ``x`` is a TypeError, bins of more than one
+    dimension or not monotonic a ValueError (reference: cunumeric/module.py:9215-9323)."""
+    x = convert_to_cunumeric_ndarray(x)
+    bins = convert_to_cunumeric_ndarray(bins)
+    if x.dtype.kind == "c":
+        raise TypeError("x may not be complex")
+    if bins.ndim > 1:
+        raise ValueError("bins must be one-dimensional")
+    b = bins.to_torch().reshape(-1)
+    increasing = bool((b[1:] >= b[:-1]).all())
+    decreasing = bool((b[1:] <= b[:-1]).all())
+    if not increasing and not decreasing:
+        raise ValueError("bins must be monotonically increasing or decreasing")
+    side = "left" if right else "right"  # backwards because the arguments are swapped
+    if increasing:
+        return searchsorted(bins, x, side=side)
+    flipped = ndarray((b.numel(),), bins.dtype, _buf=b.flip(0).contiguous().view(torch.uint8))
+    found = searchsorted(flipped, x, side=side)
+    t = found.to_torch() if isinstance(found, ndarray) else None
+    if t is None:  # scalar x
+        return int(b.numel()) - found
+    return ndarray(found.shape, np.int64, _buf=(b.numel() - t).contiguous().reshape(-1).view(torch.uint8))
 
 
 def sort(a: Any, axis: Union[int, None] = -1, kind: str = "quicksort", order=None) -> ndarray:
