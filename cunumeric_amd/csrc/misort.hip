@@ -182,7 +182,7 @@ constexpr int items_per_thread(int kb, int pay, int nt)
 #define MISORT_IPT_IDX 8
 #endif
 #ifndef MISORT_IPT_KEYS8
-#define MISORT_IPT_KEYS8 7
+#define MISORT_IPT_KEYS8 8
 #endif
   const int cap = kb <= 4 ? (pb == 8 ? 6 : (pb == 0 ? MISORT_IPT_KEYS : MISORT_IPT_IDX))
                           : (kb == 8 ? (pb == 8 ? 4 : (pb == 0 ? MISORT_IPT_KEYS8 : 7)) : (pb == 8 ? 3 : 4));

@@ -75,7 +75,8 @@ def test_twin_kernel_geometry_with_payload(nt, ipt, g, dtype):
 @pytest.mark.parametrize("kind", ["uniform", "few", "const", "ones", "runs"])
 @pytest.mark.parametrize("nt,ipt,g,n,tpc", [
     (256, 16, 32, 5 * 4096 + 77, 2),   # 4-byte keys only
-    (256, 7, 16, 9 * 1792 + 1, 4),     # 8-byte keys only
+    (256, 7, 16, 9 * 1792 + 1, 4),     # 8-byte keys only, odd keys per thread
+    (256, 8, 16, 6 * 2048 + 9, 3),     # 8-byte keys only, the kernel's keys per thread
     (256, 7, 16, 300, 4),              # a single partial tile
     (512, 3, 16, 40 * 1536 + 5, 40),   # one chunk walks many tiles: lines complete every few steps
     (256, 2, 16, 64 * 512 + 3, 16),    # two keys of a digit value per tile: the byte carry fills slowly
