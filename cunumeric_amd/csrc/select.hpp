@@ -5,7 +5,7 @@
 //   select_pick_kernel   finds the byte value whose bucket holds position kth, fixes it,
 //                        and clears the counters for the next pass.
 // After the last byte the pivot key is complete; partition / argpartition then run ONE
-// three-way split pass (upsweep / scans / downsweep with PART) around it.  The reference
+// three-way split pass (upsweep / downsweep with PART) around it.  The reference
 // sorts completely for partition (cunumeric/deferred.py:3559-3578); NumPy only asks for
 // the element at kth to be in its sorted place with nothing larger before it and nothing
 // smaller after it.
