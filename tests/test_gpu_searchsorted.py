@@ -185,3 +185,28 @@ def test_workspace_entry_point_matches_the_plain_one():
     rc = lib.misort_searchsorted_ws(code, d_a.data_ptr(), n, d_v.data_ptr(), m, 1, d_o.data_ptr(),
                                     d_s.data_ptr(), 4096, stream)
     assert rc == 4   # MISORT_ERR_SCRATCH
+
+
+@pytest.mark.parametrize("side", SIDES)
+def test_many_queries_degenerate_shapes(side):
+    """Query sets whose sorted form gives a workgroup an empty or a one-sided stretch of the
+    array: all queries equal (inside a long run of ties), all below the first element, all
+    above the last, all NaN, already sorted, reversed."""
+    rng = np.random.default_rng(73)
+    n, m = (1 << 24) + 5, (1 << 20) + 3
+    a = np.sort(np.round(rng.standard_normal(n) * 50).astype(np.float32))   # long runs of ties
+    a_num = num.array(a)
+    base = rng.standard_normal(m).astype(np.float32) * 50
+    cases = {
+        "all equal": np.full(m, 7.0, dtype=np.float32),
+        "all below": np.full(m, -1e9, dtype=np.float32),
+        "all above": np.full(m, 1e9, dtype=np.float32),
+        "all nan": np.full(m, np.nan, dtype=np.float32),
+        "sorted": np.sort(base),
+        "reversed": np.sort(base)[::-1].copy(),
+        "two far values": np.where(rng.integers(0, 2, m) == 0, np.float32(-1e9), np.float32(1e9)).astype(np.float32),
+    }
+    for name, v in cases.items():
+        print(f"searchsorted degenerate case={name} side={side}", flush=True)
+        got = np.asarray(num.searchsorted(a_num, num.array(v), side=side))
+        assert np.array_equal(got, np.searchsorted(a, v, side=side)), name
