@@ -497,7 +497,7 @@ def gpu_library_baseline(workload: str, log2n: int):
     region.  A reported comparison, like cpu_baseline; None when the program is not built or
     has no case for the workload."""
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "hipcub_calls")
-    if workload not in ("c1", "c2", "c4") or not os.access(exe, os.X_OK):
+    if workload not in ("c1", "c2", "c4", "i64small") or not os.access(exe, os.X_OK):
         return None
     import subprocess
     try:

@@ -10,9 +10,10 @@
 // The sizing calls and the allocations of the reference (a memory pool there) are made once,
 // outside the timed region, which favours the baseline.
 //
-// usage: hipcub_calls <c1|c2|c4> [log2 n] [repetitions]     prints one JSON line
+// usage: hipcub_calls <c1|c2|c4|i64small> [log2 n] [repetitions]     prints one JSON line
 //   c1: sort of int32, uniform          c2: stable argsort of float32, N(0,1) with 1 % NaN,
 //   c4: stable argsort of int64, 16 distinct values with Zipf(1.2) weights   and 1 % zeros
+//   i64small: stable argsort of int64 values below 50000
 #include <hip/hip_runtime.h>
 #include <hipcub/hipcub.hpp>
 
@@ -69,6 +70,12 @@ __global__ void gen_zipf16(int64_t* out, size_t n, const int64_t* values, const 
     while (k < 15 && u >= cdf[k]) ++k;
     out[i] = values[k];
   }
+}
+
+__global__ void gen_small_i64(int64_t* out, size_t n, uint64_t range)
+{
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    out[i] = (int64_t)(mix(i) % range);
 }
 
 __global__ void iota_i64(int64_t* out, size_t n)
@@ -159,7 +166,7 @@ int main(int argc, char** argv)
   const int lg   = argc > 2 ? std::atoi(argv[2]) : (std::strcmp(w, "c1") == 0 ? 24 : 28);
   const int reps = argc > 3 ? std::atoi(argv[3]) : 10;
   if (lg < 1 || lg > 30 || reps < 1) {
-    std::fprintf(stderr, "usage: hipcub_calls <c1|c2|c4> [log2 n <= 30] [repetitions]\n");
+    std::fprintf(stderr, "usage: hipcub_calls <c1|c2|c4|i64small> [log2 n <= 30] [repetitions]\n");
     return 2;
   }
   const size_t n = (size_t)1 << lg;
@@ -193,6 +200,11 @@ int main(int argc, char** argv)
     CHECK(hipMemcpy(dv, hv, sizeof hv, hipMemcpyHostToDevice));
     CHECK(hipMemcpy(dc, hc, sizeof hc, hipMemcpyHostToDevice));
     hipLaunchKernelGGL(gen_zipf16, dim3(4096), dim3(256), 0, 0, k, n, dv, dc);
+    run<int64_t>(w, k, n, true, reps);
+  } else if (std::strcmp(w, "i64small") == 0) {
+    int64_t* k;
+    CHECK(hipMalloc(&k, n * 8));
+    hipLaunchKernelGGL(gen_small_i64, dim3(4096), dim3(256), 0, 0, k, n, (uint64_t)50000);
     run<int64_t>(w, k, n, true, reps);
   } else {
     std::fprintf(stderr, "unknown workload %s\n", w);
