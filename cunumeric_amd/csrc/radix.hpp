@@ -121,10 +121,11 @@ struct PassPlan {
   uint32_t parity;  // dead passes before this one, modulo 2: the ping-pong buffers are swapped
   int next_shift;   // digit position of the next live pass
   int prev_live;    // the last live pass before this one
+  int const_digit;  // the digit value every key has in this pass, or -1 if the digit varies
 };
 __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
 {
-  PassPlan r{false, 0u, p.shift + RADIX_BITS, p.pass - 1};
+  PassPlan r{false, 0u, p.shift + RADIX_BITS, p.pass - 1, -1};
   if (!p.key_bits) return r;
   auto uniform64 = [](unsigned long long v) {  // same in every lane: keep it in scalar registers
     const uint32_t a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
@@ -152,6 +153,11 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
   int pv = p.pass - 1;
   while (dead(pv)) --pv;
   r.prev_live = pv;
+  {
+    const unsigned long long vary = p.pass < 8 ? lo : hi, ones = uniform64(p.pass < 8 ? w[0] : w[1]);
+    const int sh = 8 * (p.pass & 7);
+    if (((vary >> sh) & 0xFFull) == 0) r.const_digit = (int)((ones >> sh) & 0xFFull);
+  }
   return r;
 }
 // index of the ping-pong buffer that holds the input of pass p.pass (>= 1)
@@ -294,6 +300,21 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   if constexpr (!FIRST && !PART) {
     const PassPlan plan = plan_pass(p);
     if (plan.skip) return;  // every key has the same digit: the scatter of this pass is skipped too
+    if (plan.const_digit >= 0) {
+      // the last pass, which always runs, over a digit that no key varies in: the counts are
+      // the lengths of the chunks, no key needs to be read
+      const uint64_t clen = (uint64_t)p.tiles_per_chunk * p.tile, b0 = (uint64_t)chunk * clen;
+      const uint64_t b1   = b0 + clen < p.row_len ? b0 + clen : p.row_len;
+      const uint32_t cnt  = b1 > b0 ? (uint32_t)(b1 - b0) : 0u;
+      for (int d = threadIdx.x; d < RADIX; d += NT) {
+        const uint32_t c = d == plan.const_digit ? cnt : 0u;
+        p.chunk_hist[(uint64_t)blockIdx.x * RADIX + d] = c;
+        if (c)
+          atomicAdd(&p.slab_tot[((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX + d],
+                    (unsigned long long)c);
+      }
+      return;
+    }
     if (p.key_bits) p.keys_in = input_buffer(p, plan) ? p.key_buf[1] : p.key_buf[0];
     if constexpr (!SPECIALS) {
       // the last live pass wrote this pass's digits as bytes for this row: count those
