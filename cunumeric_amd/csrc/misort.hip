@@ -95,6 +95,7 @@ enum KernelId : int {
   K_SELECT_INIT,
   K_SELECT_HIST,
   K_SELECT_PICK,
+  K_SELECT_COUNTS,
   K_SPLIT,
   K_COLSORT,
   K_NUM
@@ -108,7 +109,7 @@ static const char* const kKernelNames[K_NUM] = {
   "count16_hist",    "count16_scan",    "count16_fill",     "searchsorted",
   "unique_count",    "unique_offsets",  "unique_compact",   "count8_hist",
   "count8_fill",     "select_init",     "select_hist",      "select_pick",
-  "split_downsweep", "colsort_wave"};
+  "select_counts",   "split_downsweep", "colsort_wave"};
 
 // ---------------------------------------------------------------------------------------
 // dtype table
@@ -772,6 +773,10 @@ struct PartLayout {
   bool select = false;  // false: the ordinary sort is used (it is a valid partition)
   bool by_index = false;  // values wanted but the key is not invertible: split positions, gather
   size_t off_pivot = 0, off_kleft = 0, off_ghist = 0, off_stage = 0, off_idx = 0, off_src = 0;
+  // radix select: per-row state and candidate counts, the candidate keys of every row with
+  // the chunks they came from, what every chunk counted in every pass
+  size_t off_sel_state = 0, off_cand_from = 0, off_cand_n = 0, off_cand = 0, off_cand_chunk = 0, cand_cap = 0;
+  size_t off_cand_less_eq = 0, off_pass_hist = 0, zeroed_end = 0;
   size_t total = 0;
 };
 
@@ -808,7 +813,16 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   u.off_ghist       = take(pl.rows * RADIX * sizeof(unsigned long long));
   pl.slab_tot_bytes = pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long);
   pl.off_slab_tot   = take(pl.slab_tot_bytes);  // cleared together with the counters before it
+  u.off_cand_less_eq = take(pl.n_chunks * 2 * sizeof(uint32_t));  // and with those after it
+  u.zeroed_end      = off;
   pl.off_chunk_hist = take(pl.n_chunks * RADIX * sizeof(uint32_t));
+  u.off_pass_hist   = take((size_t)dt.bytes * pl.n_chunks * RADIX * sizeof(uint32_t));
+  u.off_sel_state   = take(pl.rows * sizeof(uint32_t));
+  u.off_cand_from   = take(pl.rows * sizeof(uint32_t));
+  u.off_cand_n      = take(pl.rows * sizeof(unsigned long long));
+  u.cand_cap        = pl.row_len / 8 + 1;  // keys that still match, once they are this few
+  u.off_cand        = take(pl.rows * u.cand_cap * pl.dt.bytes);
+  u.off_cand_chunk  = take(pl.rows * u.cand_cap * sizeof(uint32_t));
   u.off_stage       = take(pl.volume * pl.dt.bytes);   // values when in == out
   u.off_idx         = take(pl.volume * sizeof(int64_t));  // positions when values are gathered
   u.off_src         = take(pl.volume * pl.dt.bytes);   // copy of the input for an in-place gather
@@ -822,29 +836,52 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
 {
   const Plan& pl     = u.pl;
   constexpr int UNT  = kUpsweepThreads;
-  KeyT* pivot        = reinterpret_cast<KeyT*>(S + u.off_pivot);
-  auto* kleft        = reinterpret_cast<unsigned long long*>(S + u.off_kleft);
-  auto* ghist        = reinterpret_cast<unsigned long long*>(S + u.off_ghist);
+  SelectParams<KeyT> sp{};
+  sp.in              = reinterpret_cast<const KeyT*>(vin);
+  sp.row_len         = pl.row_len;
+  sp.chunk_len       = (uint64_t)pl.tiles_per_chunk * pl.tile;
+  sp.chunks_per_row  = (uint32_t)pl.chunks_per_row;
+  sp.n_chunks        = (uint32_t)pl.n_chunks;
+  sp.n_passes        = (uint32_t)sizeof(KeyT);
+  sp.xform           = pl.dt.xform;
+  sp.prefix          = reinterpret_cast<KeyT*>(S + u.off_pivot);
+  sp.kleft           = reinterpret_cast<unsigned long long*>(S + u.off_kleft);
+  sp.ghist           = reinterpret_cast<unsigned long long*>(S + u.off_ghist);
+  sp.pass_hist       = reinterpret_cast<uint32_t*>(S + u.off_pass_hist);
+  sp.state           = reinterpret_cast<uint32_t*>(S + u.off_sel_state);
+  sp.cand_from       = reinterpret_cast<uint32_t*>(S + u.off_cand_from);
+  sp.cand            = reinterpret_cast<KeyT*>(S + u.off_cand);
+  sp.cand_chunk      = reinterpret_cast<uint32_t*>(S + u.off_cand_chunk);
+  sp.cand_n          = reinterpret_cast<unsigned long long*>(S + u.off_cand_n);
+  sp.cand_cap        = u.cand_cap;
+  sp.cand_less_eq    = reinterpret_cast<uint32_t*>(S + u.off_cand_less_eq);
+  sp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
+  sp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
+  sp.chunks_per_slab = (uint32_t)pl.chunks_per_slab;
+  sp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
+  KeyT* pivot        = sp.prefix;
   const dim3 grid((unsigned)pl.n_chunks);
   const dim3 rgrid((unsigned)pl.rows);
-  const uint64_t clen = (uint64_t)pl.tiles_per_chunk * pl.tile;
 
-  launch_zero(L, ghist, pl.off_slab_tot + pl.slab_tot_bytes - u.off_ghist);
+  launch_zero(L, sp.ghist, u.zeroed_end - u.off_ghist);
   L.run(K_SELECT_INIT, [&] {
     hipLaunchKernelGGL((select_init_kernel<KeyT>), dim3((unsigned)((pl.rows + 255) / 256)), dim3(256), 0,
-                       L.stream, pivot, kleft, (uint32_t)pl.rows, (unsigned long long)kth);
+                       L.stream, sp, (uint32_t)pl.rows, (unsigned long long)kth);
   });
-  for (int shift = (int)sizeof(KeyT) * 8 - 8; shift >= 0; shift -= 8) {
+  int pass = 0;
+  for (int shift = (int)sizeof(KeyT) * 8 - 8; shift >= 0; shift -= 8, ++pass) {
     L.run(K_SELECT_HIST, [&] {
-      hipLaunchKernelGGL((select_hist_kernel<KeyT>), grid, dim3(SEL_NT), 0, L.stream,
-                         reinterpret_cast<const KeyT*>(vin), (uint64_t)pl.row_len, clen,
-                         (uint32_t)pl.chunks_per_row, pl.dt.xform, shift, pivot, ghist);
+      hipLaunchKernelGGL((select_hist_kernel<KeyT>), grid, dim3(SEL_NT), 0, L.stream, sp, pass, shift);
     });
     L.run(K_SELECT_PICK, [&] {
-      hipLaunchKernelGGL((select_pick_kernel<KeyT>), rgrid, dim3(RADIX), 0, L.stream, pivot, kleft,
-                         ghist, shift);
+      hipLaunchKernelGGL((select_pick_kernel<KeyT>), rgrid, dim3(RADIX), 0, L.stream, sp, pass, shift);
     });
   }
+  // the counts the split pass needs, from what the passes above counted per chunk
+  L.run(K_SELECT_COUNTS, [&] {
+    hipLaunchKernelGGL((select_cand_counts_kernel<KeyT>), grid, dim3(SEL_NT), 0, L.stream, sp);
+    hipLaunchKernelGGL((select_chunk_counts_kernel<KeyT>), grid, dim3(RADIX), 0, L.stream, sp);
+  });
 
   PassParams pp{};
   pp.keys_in         = vin;
@@ -865,9 +902,6 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.xform           = pl.dt.xform;
   pp.shift           = 0;
   pp.pivot           = pivot;
-  L.run(K_UPSWEEP, [&] {
-    hipLaunchKernelGGL((upsweep_kernel<KeyT, true, false, UNT, true>), grid, dim3(UNT), 0, L.stream, pp);
-  });
   launch_downsweep<KeyT, PAY, true>(L, pl, K_SPLIT, true, true, pp);
 }
 

@@ -4,12 +4,21 @@
 //                        fixed so far (one read of the row),
 //   select_pick_kernel   finds the byte value whose bucket holds position kth, fixes it,
 //                        and clears the counters for the next pass.
+// Once the keys that still match are few (at most an eighth of the row, known after a pick),
+// the next histogram pass also writes them out side by side ("candidates"), and the passes
+// after that read the candidates instead of the row: with uniform keys the last two of four
+// passes then read 1/256 of the data.  The state of a row (SEL_ROW / SEL_APPEND / SEL_CAND)
+// lives on the device and is advanced by select_pick_kernel.
 // After the last byte the pivot key is complete; partition / argpartition then run ONE
-// three-way split pass (upsweep / downsweep with PART) around it.  The reference
+// three-way split pass (the downsweep with PART) around it.  The counts that pass needs per
+// chunk (keys below / equal to / above the pivot) are put together from what the chunks
+// counted during the selection (select_cand_counts_kernel, select_chunk_counts_kernel), so
+// the row is not read once more to count them.  The reference
 // sorts completely for partition (cunumeric/deferred.py:3559-3578); NumPy only asks for
 // the element at kth to be in its sorted place with nothing larger before it and nothing
 // smaller after it.
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -19,6 +28,8 @@
 namespace misort {
 
 constexpr int SEL_NT = 256;
+// where the histogram pass of a row reads its keys, and whether it writes candidates
+constexpr uint32_t SEL_ROW = 0, SEL_APPEND = 1, SEL_CAND = 2;
 
 // do the bytes of k above bit position `shift + 8` equal those of the prefix?
 template <typename KeyT>
@@ -45,48 +56,131 @@ __device__ __forceinline__ KeyT select_with_byte(KeyT prefix, uint32_t b, int sh
   }
 }
 
-// grid: rows * chunks_per_row; the chunk geometry is the one of the split pass that follows
+// What the kernels of a selection share.  All arrays live in the caller's scratch memory.
 template <typename KeyT>
-__global__ void __launch_bounds__(SEL_NT)
-select_hist_kernel(const KeyT* __restrict__ in, uint64_t row_len, uint64_t chunk_len,
-                   uint32_t chunks_per_row, int xform, int shift, const KeyT* __restrict__ prefix,
-                   unsigned long long* __restrict__ ghist)
+struct SelectParams {
+  const KeyT* in;                 // rows of row_len values
+  uint64_t row_len, chunk_len;    // chunk geometry: the one of the split pass that follows
+  uint32_t chunks_per_row, n_chunks, n_passes;
+  int xform;
+  KeyT* prefix;                   // per row: the bytes of the kth key found so far
+  unsigned long long* kleft;      // per row: position of kth among the keys that match the prefix
+  unsigned long long* ghist;      // per row: RADIX counters of the current pass
+  uint32_t* pass_hist;            // [pass][chunk][RADIX]: what each chunk counted when it read the row
+  uint32_t* state;                // per row: SEL_ROW / SEL_APPEND / SEL_CAND
+  uint32_t* cand_from;            // per row: first pass that read the candidates (n_passes: none did)
+  KeyT* cand;                     // per row: cand_cap keys (transformed)
+  uint32_t* cand_chunk;           // the chunk each candidate came from
+  unsigned long long* cand_n;     // per row: candidates written
+  uint64_t cand_cap;
+  uint32_t* cand_less_eq;         // per chunk: candidates below the kth key, and equal to it
+  // outputs for the split pass (what its own counting pass would have written)
+  uint32_t* chunk_hist;           // [chunk][RADIX]: keys below / equal / above in 0 / 1 / 2
+  unsigned long long* slab_tot;   // [row][slab][RADIX], zero on entry
+  uint32_t chunks_per_slab, slabs_per_row;
+};
+
+// grid: n_chunks.  Pass `pass` counts byte `shift / 8` of the keys that match the prefix.
+// state[row]: SEL_ROW reads the row; SEL_APPEND reads the row and appends the keys that match
+// the prefix to the row's candidates; SEL_CAND reads those candidates (they are keys already),
+// spread evenly over the row's workgroups.
+template <typename KeyT>
+__global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> p, int pass, int shift)
 {
   constexpr int NW = SEL_NT / 64, COPIES = 4;
+  // Candidates are collected per wavefront and written out a few hundred at a time: the
+  // place in the row's candidate area comes from one counter, and atomics on one address
+  // queue up, so there must be few of them.
+  constexpr uint32_t CB = 4096 / sizeof(KeyT);
   __shared__ __attribute__((aligned(16))) uint32_t h[NW * RADIX * COPIES];
+  __shared__ __attribute__((aligned(16))) KeyT cbuf[NW * CB];
   for (int i = threadIdx.x; i < NW * RADIX * COPIES; i += SEL_NT) h[i] = 0;
   __syncthreads();
-  const uint32_t row = blockIdx.x / chunks_per_row, chunk = blockIdx.x % chunks_per_row;
+  const uint32_t row = blockIdx.x / p.chunks_per_row, chunk = blockIdx.x % p.chunks_per_row;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t* my     = h + wave * (RADIX * COPIES) + (lane & (COPIES - 1));
-  const KeyT pre   = prefix[row];
-  const KeyT* base = in + (uint64_t)row * row_len;
-  const uint64_t b0 = (uint64_t)chunk * chunk_len;
-  uint64_t b1       = b0 + chunk_len;
-  if (b1 > row_len) b1 = row_len;
-  auto count = [&](KeyT raw) {
-    const KeyT k = KeyOps<KeyT>::to_key(raw, xform);
-    if (select_matches(k, pre, shift)) atomicAdd(&my[KeyOps<KeyT>::digit(k, shift) * COPIES], 1u);
-  };
-  // 16-byte loads where the row allows it
+  uint32_t* my      = h + wave * (RADIX * COPIES) + (lane & (COPIES - 1));
+  const KeyT pre    = p.prefix[row];
+  const uint32_t st = p.state[row];
+  KeyT* my_cand     = p.cand + (uint64_t)row * p.cand_cap;
+  const KeyT* base;
+  uint64_t b0, b1;
+  if (st == SEL_CAND) {
+    const uint64_t n_c = p.cand_n[row];
+    const uint64_t per = (n_c + p.chunks_per_row - 1) / p.chunks_per_row;
+    base = my_cand;
+    b0   = (uint64_t)chunk * per;
+    b1   = b0 + per < n_c ? b0 + per : n_c;
+    if (b0 > b1) b0 = b1;
+  } else {
+    base = p.in + (uint64_t)row * p.row_len;
+    b0   = (uint64_t)chunk * p.chunk_len;
+    b1   = b0 + p.chunk_len;
+    if (b1 > p.row_len) b1 = p.row_len;
+    if (b0 > b1) b0 = b1;
+  }
   constexpr int V = sizeof(KeyT) >= 16 ? 1 : 16 / sizeof(KeyT);
   struct alignas(16) Vec {
     KeyT v[V];
   };
-  uint64_t i0 = b0;
-  if (V > 1 && (reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
-    const uint64_t nvec = (b1 - b0) / V;
-    const Vec* vb       = reinterpret_cast<const Vec*>(base + b0);
-    if constexpr (sizeof(Vec) == 16) {
-      stream_vectors<4>(vb, nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
+  // (one instance of the loop per state, so that the plain pass carries none of the rest)
+  auto scan = [&](auto state_tag) {
+    constexpr uint32_t ST = decltype(state_tag)::value;
+    uint32_t n_buf        = 0;  // APPEND: keys in this wavefront's part of cbuf (same in every lane)
+    KeyT* wbuf            = cbuf + wave * CB;
+    auto flush = [&] {
+      unsigned long long at = 0;
+      if (lane == 0) at = atomicAdd(&p.cand_n[row], (unsigned long long)n_buf);
+      at = __shfl(at, 0, 64);
+      for (uint32_t i = lane; i < n_buf; i += 64) {
+        my_cand[at + i]                                     = wbuf[i];
+        p.cand_chunk[(uint64_t)row * p.cand_cap + at + i] = blockIdx.x;
+      }
+      n_buf = 0;
+    };
+    // APPEND calls this with all lanes of the wavefront present; `valid` marks the real keys
+    auto count = [&](KeyT raw, bool valid) {
+      const KeyT k     = ST == SEL_CAND ? raw : KeyOps<KeyT>::to_key(raw, p.xform);
+      const bool match = valid && select_matches(k, pre, shift);
+      if (match) atomicAdd(&my[KeyOps<KeyT>::digit(k, shift) * COPIES], 1u);
+      if constexpr (ST == SEL_APPEND) {
+        const uint64_t m = __ballot(match);
+        if (m) {
+          if (match) wbuf[n_buf + __popcll(m & ((1ull << lane) - 1))] = k;
+          n_buf += __popcll(m);
+          if (n_buf > CB - 64) flush();
+        }
+      }
+    };
+    // 16-byte loads where the row allows it; in whole batches only when appending, so that the
+    // rest is done with the wavefronts intact
+    uint64_t i0 = b0;
+    if (V > 1 && (reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
+      uint64_t nvec = (b1 - b0) / V;
+      if (ST == SEL_APPEND) nvec -= nvec % ((uint64_t)SEL_NT * 4);
+      const Vec* vb = reinterpret_cast<const Vec*>(base + b0);
+      if constexpr (sizeof(Vec) == 16) {
+        stream_vectors<4>(vb, nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) count(r.v[e]);
-      });
+          for (int e = 0; e < V; ++e) count(r.v[e], true);
+        });
+      }
+      i0 = b0 + nvec * V;
     }
-    i0 = b0 + nvec * V;
-  }
-  for (uint64_t i = i0 + threadIdx.x; i < b1; i += SEL_NT) count(base[i]);
+    if constexpr (ST == SEL_APPEND) {
+      for (uint64_t i = i0; i < b1; i += SEL_NT) {  // the same number of rounds for every lane
+        const bool valid = i + threadIdx.x < b1;
+        count(valid ? base[i + threadIdx.x] : KeyT{}, valid);
+      }
+      if (n_buf) flush();
+    } else {
+      for (uint64_t i = i0 + threadIdx.x; i < b1; i += SEL_NT) count(base[i], true);
+    }
+  };
+  if (st == SEL_ROW) scan(std::integral_constant<uint32_t, SEL_ROW>{});
+  else if (st == SEL_APPEND) scan(std::integral_constant<uint32_t, SEL_APPEND>{});
+  else scan(std::integral_constant<uint32_t, SEL_CAND>{});
   __syncthreads();
+  uint32_t* mine = p.pass_hist + ((uint64_t)pass * p.n_chunks + blockIdx.x) * RADIX;
   for (int d = threadIdx.x; d < RADIX; d += SEL_NT) {
     uint32_t c = 0;
 #pragma unroll
@@ -94,44 +188,147 @@ select_hist_kernel(const KeyT* __restrict__ in, uint64_t row_len, uint64_t chunk
       const uint4 q = *reinterpret_cast<const uint4*>(&h[(w * RADIX + d) * COPIES]);
       c += q.x + q.y + q.z + q.w;
     }
-    if (c) atomicAdd(&ghist[(uint64_t)row * RADIX + d], (unsigned long long)c);
+    if (c) atomicAdd(&p.ghist[(uint64_t)row * RADIX + d], (unsigned long long)c);
+    if (st != SEL_CAND) mine[d] = c;
   }
 }
 
-// grid: rows, RADIX threads.  kleft[row] = position of kth among the keys that match the prefix.
+// grid: rows, RADIX threads.  Finds the byte value whose keys include position kleft[row].
+// Also advances the row's state: a pass that appended is followed by passes over the
+// candidates; a row whose chosen bucket fits the candidate area (and that has two more passes
+// to go, so that one of them profits) appends in its next pass.
 template <typename KeyT>
-__global__ void __launch_bounds__(RADIX)
-select_pick_kernel(KeyT* __restrict__ prefix, unsigned long long* __restrict__ kleft,
-                   unsigned long long* __restrict__ ghist, int shift)
+__global__ void __launch_bounds__(RADIX) select_pick_kernel(SelectParams<KeyT> p, int pass, int shift)
 {
   __shared__ unsigned long long wave_tot[RADIX / 64];
   const uint32_t row = blockIdx.x;
   const int d = threadIdx.x, lane = d & 63, wave = d >> 6;
-  unsigned long long* g      = ghist + (uint64_t)row * RADIX;
+  unsigned long long* g      = p.ghist + (uint64_t)row * RADIX;
   const unsigned long long c = g[d];
   g[d]                       = 0;  // ready for the next pass
   const unsigned long long incl = wave_incl_scan(c, lane);
   if (lane == 63) wave_tot[wave] = incl;
-  const unsigned long long k = kleft[row];
+  const unsigned long long k = p.kleft[row];
   __syncthreads();
   unsigned long long before = incl - c;
   for (int w = 0; w < wave; ++w) before += wave_tot[w];
   if (c != 0 && before <= k && k < before + c) {  // exactly one thread
-    prefix[row] = select_with_byte(prefix[row], (uint32_t)d, shift);
-    kleft[row]  = k - before;
+    p.prefix[row] = select_with_byte(p.prefix[row], (uint32_t)d, shift);
+    p.kleft[row]  = k - before;
+    const uint32_t st = p.state[row];
+    if (st == SEL_APPEND) {
+      p.state[row]     = SEL_CAND;
+      p.cand_from[row] = (uint32_t)pass + 1;
+    } else if (st == SEL_ROW && c <= p.cand_cap && shift >= 16) {
+      p.state[row] = SEL_APPEND;
+    }
   }
 }
 
-// grid-stride: prefix <- 0, kleft <- kth
+// grid-stride: prefix <- 0, kleft <- kth, the row is read, no candidates yet
 template <typename KeyT>
-__global__ void __launch_bounds__(256)
-select_init_kernel(KeyT* __restrict__ prefix, unsigned long long* __restrict__ kleft, uint32_t rows,
-                   unsigned long long kth)
+__global__ void __launch_bounds__(256) select_init_kernel(SelectParams<KeyT> p, uint32_t rows, unsigned long long kth)
 {
   for (uint32_t r = blockIdx.x * 256 + threadIdx.x; r < rows; r += gridDim.x * 256) {
-    prefix[r] = KeyT{};
-    kleft[r]  = kth;
+    p.prefix[r]    = KeyT{};
+    p.kleft[r]     = kth;
+    p.state[r]     = SEL_ROW;
+    p.cand_from[r] = p.n_passes;
+    p.cand_n[r]    = 0;
   }
+}
+
+// grid: n_chunks, after the last pick.  Of the candidates of a row that ended up reading
+// them, those that share the bytes of the kth key up to the pass that wrote them (the others
+// were told apart by that pass's own count) are compared with the kth key, and the chunk
+// each came from gets them added to its "below" or "equal" count (cand_less_eq, zero on entry).
+template <typename KeyT>
+__global__ void __launch_bounds__(SEL_NT) select_cand_counts_kernel(SelectParams<KeyT> p)
+{
+  const uint32_t row = blockIdx.x / p.chunks_per_row, chunk = blockIdx.x % p.chunks_per_row;
+  const uint32_t from = p.cand_from[row];
+  if (from >= p.n_passes) return;
+  const int lane = threadIdx.x & 63;
+  const KeyT kth      = p.prefix[row];
+  const int low_shift = (int)sizeof(KeyT) * 8 - 8 * (int)from - 8;  // the first pass over the candidates
+  const uint64_t n_c  = p.cand_n[row];
+  const uint64_t per  = (n_c + p.chunks_per_row - 1) / p.chunks_per_row;
+  uint64_t b0 = (uint64_t)chunk * per, b1 = b0 + per < n_c ? b0 + per : n_c;
+  const KeyT* cand    = p.cand + (uint64_t)row * p.cand_cap;
+  const uint32_t* src = p.cand_chunk + (uint64_t)row * p.cand_cap;
+  for (uint64_t i0 = b0; i0 < b1; i0 += SEL_NT) {  // the same number of rounds for every lane
+    const uint64_t i = i0 + threadIdx.x;
+    bool less = false, equal = false;
+    uint32_t c = 0;
+    if (i < b1) {
+      const KeyT k = cand[i];
+      c            = src[i];
+      if (select_matches(k, kth, low_shift)) {
+        less  = key_lt(k, kth);
+        equal = key_eq(k, kth);
+      }
+    }
+    // candidates of one chunk lie together in runs, so mostly the whole wavefront adds to one chunk
+    const uint64_t any = __ballot(less || equal);
+    if (any == 0) continue;
+    const uint32_t c0 = __shfl(c, __builtin_ctzll(any), 64);
+    if (__ballot((less || equal) && c != c0) == 0) {
+      const uint32_t nl = __popcll(__ballot(less)), ne = __popcll(__ballot(equal));
+      if (lane == 0) {
+        if (nl) atomicAdd(&p.cand_less_eq[2 * (uint64_t)c0], nl);
+        if (ne) atomicAdd(&p.cand_less_eq[2 * (uint64_t)c0 + 1], ne);
+      }
+    } else if (less || equal) {
+      atomicAdd(&p.cand_less_eq[2 * (uint64_t)c + (equal ? 1 : 0)], 1u);
+    }
+  }
+}
+
+// grid: n_chunks, RADIX threads, after select_cand_counts_kernel.  Puts together, per chunk,
+// how many of its keys lie below the kth key, equal it, and lie above, from what the chunk
+// counted in the passes that read the row (a key is below if, at the first byte where it
+// leaves the kth key, its byte is smaller) and from its candidates; written in the form the
+// split pass expects from a counting pass of its own, which therefore does not run.
+template <typename KeyT>
+__global__ void __launch_bounds__(RADIX) select_chunk_counts_kernel(SelectParams<KeyT> p)
+{
+  __shared__ unsigned long long wave_tot[RADIX / 64];
+  const uint32_t row = blockIdx.x / p.chunks_per_row, chunk = blockIdx.x % p.chunks_per_row;
+  const int d = threadIdx.x, lane = d & 63, wave = d >> 6;
+  const uint32_t from = p.cand_from[row];
+  const KeyT kth      = p.prefix[row];
+  unsigned long long below = 0;
+  uint32_t equal           = 0;
+  for (uint32_t q = 0; q < from; ++q) {
+    const int shift   = (int)sizeof(KeyT) * 8 - 8 - 8 * (int)q;
+    const uint32_t kb = KeyOps<KeyT>::digit(kth, shift);
+    const uint32_t c  = p.pass_hist[((uint64_t)q * p.n_chunks + blockIdx.x) * RADIX + d];
+    if ((uint32_t)d < kb) below += c;
+    if (q + 1 == p.n_passes && (uint32_t)d == kb) equal = c;  // only one thread
+  }
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) {
+    below += __shfl_xor(below, s, 64);
+    equal += __shfl_xor(equal, s, 64);
+  }
+  if (lane == 0) wave_tot[wave] = (below << 32) | equal;  // a chunk has fewer than 2^32 keys
+  __syncthreads();
+  unsigned long long t = 0;
+  for (int w = 0; w < RADIX / 64; ++w) t += wave_tot[w];  // (the halves do not carry into each other)
+  uint32_t n_below = (uint32_t)(t >> 32), n_equal = (uint32_t)t;
+  if (from < p.n_passes) {
+    n_below += p.cand_less_eq[2 * (uint64_t)blockIdx.x];
+    n_equal = p.cand_less_eq[2 * (uint64_t)blockIdx.x + 1];
+  }
+  uint64_t b0 = (uint64_t)chunk * p.chunk_len, b1 = b0 + p.chunk_len;
+  if (b1 > p.row_len) b1 = p.row_len;
+  if (b0 > b1) b0 = b1;
+  const uint32_t len = (uint32_t)(b1 - b0);
+  const uint32_t c   = d == 0 ? n_below : d == 1 ? n_equal : d == 2 ? len - n_below - n_equal : 0u;
+  p.chunk_hist[(uint64_t)blockIdx.x * RADIX + d] = c;
+  if (c)
+    atomicAdd(&p.slab_tot[((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX + d],
+              (unsigned long long)c);
 }
 
 }  // namespace misort

@@ -80,6 +80,32 @@ def test_rows_axes_and_fallbacks():
     assert np.array_equal(np.asarray(num.partition(d, 10**9)), np.sort(d))
 
 
+@pytest.mark.parametrize("dtype", [np.uint32, np.int64, np.float64], ids=lambda d: np.dtype(d).name)
+def test_rows_that_narrow_down_at_different_passes(dtype):
+    """The selection writes the keys that still match side by side once they are few and reads
+    only those afterwards; when that happens depends on the row: at once (all bytes vary), after
+    some passes (leading bytes equal), never (few distinct values), or only for some ranks
+    (one heavy value beside spread-out ones)."""
+    rng = np.random.default_rng(54)
+    n = 300007
+    bits = np.dtype(dtype).itemsize * 8
+    rows = [
+        rng.integers(0, 2**(bits - 1), n, dtype=np.uint64),            # every byte varies
+        rng.integers(0, 2**16, n, dtype=np.uint64) + (1 << (bits - 3)),  # only the low two bytes
+        rng.integers(0, 2**24, n, dtype=np.uint64) << np.uint64(8),     # the lowest byte is constant
+        rng.integers(0, 3, n, dtype=np.uint64) * 77,                     # three values
+        np.where(rng.random(n) < 0.6, 12345, rng.integers(0, 2**(bits - 1), n, dtype=np.uint64)),
+    ]
+    a = np.stack(rows).astype(np.uint64)
+    a = a.astype(dtype) if np.dtype(dtype).kind != "f" else (a.astype(np.float64) - 2.0**40)
+    for kth in (0, 7, n // 5, n // 2, n - 2):
+        print(f"narrowing dtype={np.dtype(dtype).name} kth={kth}", flush=True)
+        assert_partitioned(a, num.partition(a, kth, axis=1), kth)
+        idx = np.asarray(num.argpartition(a, kth, axis=1))
+        assert np.array_equal(np.sort(idx, axis=1), np.broadcast_to(np.arange(n), a.shape))
+        assert_partitioned(a, np.take_along_axis(a, idx, axis=1), kth)
+
+
 def test_c_abi_plan_and_offset(abi):
     """the C entry point directly: positions carry index_offset; 2-byte values still count"""
     import torch
