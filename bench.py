@@ -398,6 +398,77 @@ def run_partition(args) -> int:
     return 0 if ok else 1
 
 
+def run_select(args) -> int:
+    """--workload sel: the two middle order statistics and the largest element of 2^log2n
+    float32 (the C2 input) by selection, which is what quantile / percentile / median need of
+    the sort (the reference sorts the array for them; not the headline)."""
+    import torch
+
+    import cunumeric_amd as num
+    from cunumeric_amd import _lib
+    from cunumeric_amd.config import to_core_dtype
+
+    lib = _lib.load()
+    dev = torch.device("cuda", 0)
+    log2n = args.log2n if args.log2n is not None else 28
+    n = 1 << log2n
+    kth = n // 2 - 1
+    a = make_c2(n, seed=2)
+    d_a = torch.from_numpy(a.view(np.uint8)).to(dev)
+    d_o = torch.zeros(3 * 4, dtype=torch.uint8, device=dev)
+    code = to_core_dtype(np.float32)
+    need = lib.misort_select_scratch_bytes(code, n, n, kth)
+    scratch = torch.empty(need, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        _lib.check(lib.misort_select(code, d_a.data_ptr(), n, n, kth, d_o.data_ptr(), d_o.data_ptr() + 4,
+                                     d_o.data_ptr() + 8, scratch.data_ptr(), need, stream))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    got = d_o.cpu().numpy().view(np.float32)
+    sample = a[: 1 << 25]
+    t1 = time.perf_counter()
+    np.partition(sample, [sample.size // 2 - 1, sample.size // 2])
+    cpu = sample.size / (time.perf_counter() - t1) / 1e9
+    ref = np.partition(a, [kth, kth + 1])  # NaNs order last in NumPy too
+    ok = bool(got[0] == ref[kth]) and bool(got[1] == ref[kth + 1]) and bool(np.isnan(got[2]))
+    # the Python caller, end to end (allocations, the blend and the NaN test through torch)
+    d_arr = num.array(a)
+    med = float(np.asarray(num.quantile(d_arr, 0.5)))
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for _ in range(args.steps):
+        num.quantile(d_arr, 0.5)
+    torch.cuda.synchronize()
+    dq = (time.perf_counter() - t2) / args.steps
+    ok = ok and np.isnan(med)  # the input holds NaNs: no quantile, as in NumPy
+    b = 2 * 4  # two selection passes over the row (the rest reads the few keys that still match)
+    out = {
+        "metric": f"Gkeys/s, elements kth, kth+1 and last in sort order of 2^{log2n} float32, 1 MI355X",
+        "value": n / dt / 1e9, "unit": "Gkeys/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {"workload": f"select, float32 (C2 input), n=2^{log2n}, kth=n/2-1"},
+        "parity_guard": "ok" if ok else "FAILED",
+        "quantile_call_ms": dq * 1e3,
+        "roofline": {"bound": "hbm", "kernel": "select_hist", "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "achieved": b * n / dt / 1e9, "frac": b * n / dt / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "note": "whole call, 8 algorithmic bytes per key"},
+        "cpu_baseline": {"value": cpu, "unit": "Gkeys/s", "cores": 1, "kind": "port",
+                         "sample": "numpy.partition around the two middle positions of the first 2^25 elements"},
+    }
+    print(json.dumps(out))
+    return 0 if ok else 1
+
+
 def run_axis(args) -> int:
     """--workload axis: sort of a float32 (k, 2^log2n / k) array along axis 0, k = 256: the
     column kernel, with the transposed route (swap, row sort, swap: what the reference does)
@@ -518,7 +589,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ss", "uniq", "part", "axis"], default="c2")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ss", "uniq", "part", "sel", "axis"], default="c2")
     ap.add_argument("--log2n", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true")
@@ -546,6 +617,8 @@ def main() -> int:
         return run_axis(args)
     if args.workload == "part":
         return run_partition(args)
+    if args.workload == "sel":
+        return run_select(args)
     dev = torch.device("cuda", 0)
     title, gen, def_log2n, argsort, row = WORKLOADS[args.workload]
     log2n = args.log2n if args.log2n is not None else def_log2n

@@ -34,6 +34,8 @@ EXPORTS = (
     "misort_unique",
     "misort_partition_scratch_bytes",
     "misort_partition",
+    "misort_select_scratch_bytes",
+    "misort_select",
     "misort_sort_axis",
 )
 
@@ -121,6 +123,11 @@ def load():
     lib.misort_partition.restype = c_int
     lib.misort_partition.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t,
                                      ctypes.c_longlong, c_int64, c_void_p, c_size_t, c_void_p]
+    lib.misort_select_scratch_bytes.restype = c_size_t
+    lib.misort_select_scratch_bytes.argtypes = [c_int, c_size_t, c_size_t, ctypes.c_longlong]
+    lib.misort_select.restype = c_int
+    lib.misort_select.argtypes = [c_int, c_void_p, c_size_t, c_size_t, ctypes.c_longlong, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_size_t, c_void_p]
     lib.misort_sort_axis.restype = c_int
     lib.misort_sort_axis.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_size_t,
                                      c_int64, c_void_p]

@@ -96,6 +96,8 @@ enum KernelId : int {
   K_SELECT_HIST,
   K_SELECT_PICK,
   K_SELECT_COUNTS,
+  K_SELECT_NEIGHBOURS,
+  K_SELECT_EMIT,
   K_SPLIT,
   K_COLSORT,
   K_NUM
@@ -109,7 +111,8 @@ static const char* const kKernelNames[K_NUM] = {
   "count16_hist",    "count16_scan",    "count16_fill",     "searchsorted",
   "unique_count",    "unique_offsets",  "unique_compact",   "count8_hist",
   "count8_fill",     "select_init",     "select_hist",      "select_pick",
-  "select_counts",   "split_downsweep", "colsort_wave"};
+  "select_counts",   "select_above",    "select_emit",    "split_downsweep",
+  "colsort_wave"};
 
 // ---------------------------------------------------------------------------------------
 // dtype table
@@ -777,16 +780,18 @@ struct PartLayout {
   // the chunks they came from, what every chunk counted in every pass
   size_t off_sel_state = 0, off_cand_from = 0, off_cand_n = 0, off_cand = 0, off_cand_chunk = 0, cand_cap = 0;
   size_t off_cand_less_eq = 0, off_pass_hist = 0, zeroed_end = 0;
+  size_t off_n_equal = 0, off_above_max = 0;
   size_t total = 0;
 };
 
+// select_only: the layout of misort_select, which finds the key and does not move the row
 static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool want_indices,
-                            long long kth, PartLayout& u)
+                            long long kth, PartLayout& u, bool select_only = false)
 {
   DtypeInfo dt;
   if (!dtype_info(dtype, dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
   const bool lossy = dt.xform == XF_FLOAT || dt.xform == XF_COMPLEX;  // key does not keep all bits
-  u.by_index       = !want_indices && lossy;
+  u.by_index       = !want_indices && lossy && !select_only;
   int rc = make_plan(dtype, volume, sort_dim_size, want_indices || u.by_index, false, u.pl);
   if (rc != MISORT_OK) return rc;
   // 1- and 2-byte values are counted, which beats selecting; their positions are selected
@@ -818,24 +823,29 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   pl.off_chunk_hist = take(pl.n_chunks * RADIX * sizeof(uint32_t));
   u.off_pass_hist   = take((size_t)dt.bytes * pl.n_chunks * RADIX * sizeof(uint32_t));
   u.off_sel_state   = take(pl.rows * sizeof(uint32_t));
+  u.off_n_equal     = take(pl.rows * sizeof(unsigned long long));
+  u.off_above_max   = take(pl.rows * 2 * sizeof(unsigned long long));
   u.off_cand_from   = take(pl.rows * sizeof(uint32_t));
   u.off_cand_n      = take(pl.rows * sizeof(unsigned long long));
   u.cand_cap        = pl.row_len / 8 + 1;  // keys that still match, once they are this few
   u.off_cand        = take(pl.rows * u.cand_cap * pl.dt.bytes);
   u.off_cand_chunk  = take(pl.rows * u.cand_cap * sizeof(uint32_t));
-  u.off_stage       = take(pl.volume * pl.dt.bytes);   // values when in == out
-  u.off_idx         = take(pl.volume * sizeof(int64_t));  // positions when values are gathered
-  u.off_src         = take(pl.volume * pl.dt.bytes);   // copy of the input for an in-place gather
-  u.total           = off;
+  if (!select_only) {
+    u.off_stage = take(pl.volume * pl.dt.bytes);      // values when in == out
+    u.off_idx   = take(pl.volume * sizeof(int64_t));  // positions when values are gathered
+    u.off_src   = take(pl.volume * pl.dt.bytes);      // copy of the input for an in-place gather
+  }
+  u.total = off;
   return MISORT_OK;
 }
 
-template <typename KeyT, int PAY>
-static void partition_select_rows(Launcher& L, const PartLayout& u, const void* vin, void* keys_out,
-                                  void* pay_out, long long kth, int64_t index_offset, char* S)
+// The selection proper: after it sp.prefix holds the kth key of every row.  neighbours: the
+// rows' above_max words are wanted (select_init_kernel sets them up).
+template <typename KeyT>
+static SelectParams<KeyT> run_selection(Launcher& L, const PartLayout& u, const void* vin, long long kth,
+                                        char* S, bool neighbours)
 {
-  const Plan& pl     = u.pl;
-  constexpr int UNT  = kUpsweepThreads;
+  const Plan& pl = u.pl;
   SelectParams<KeyT> sp{};
   sp.in              = reinterpret_cast<const KeyT*>(vin);
   sp.row_len         = pl.row_len;
@@ -854,12 +864,13 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   sp.cand_chunk      = reinterpret_cast<uint32_t*>(S + u.off_cand_chunk);
   sp.cand_n          = reinterpret_cast<unsigned long long*>(S + u.off_cand_n);
   sp.cand_cap        = u.cand_cap;
+  sp.n_equal         = reinterpret_cast<unsigned long long*>(S + u.off_n_equal);
+  sp.above_max       = neighbours ? reinterpret_cast<unsigned long long*>(S + u.off_above_max) : nullptr;
   sp.cand_less_eq    = reinterpret_cast<uint32_t*>(S + u.off_cand_less_eq);
   sp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
   sp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
   sp.chunks_per_slab = (uint32_t)pl.chunks_per_slab;
   sp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
-  KeyT* pivot        = sp.prefix;
   const dim3 grid((unsigned)pl.n_chunks);
   const dim3 rgrid((unsigned)pl.rows);
 
@@ -877,6 +888,16 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
       hipLaunchKernelGGL((select_pick_kernel<KeyT>), rgrid, dim3(RADIX), 0, L.stream, sp, pass, shift);
     });
   }
+  return sp;
+}
+
+template <typename KeyT, int PAY>
+static void partition_select_rows(Launcher& L, const PartLayout& u, const void* vin, void* keys_out,
+                                  void* pay_out, long long kth, int64_t index_offset, char* S)
+{
+  const Plan& pl              = u.pl;
+  const SelectParams<KeyT> sp = run_selection<KeyT>(L, u, vin, kth, S, false);
+  const dim3 grid((unsigned)pl.n_chunks);
   // the counts the split pass needs, from what the passes above counted per chunk
   L.run(K_SELECT_COUNTS, [&] {
     hipLaunchKernelGGL((select_cand_counts_kernel<KeyT>), grid, dim3(SEL_NT), 0, L.stream, sp);
@@ -901,8 +922,30 @@ static void partition_select_rows(Launcher& L, const PartLayout& u, const void* 
   pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
   pp.xform           = pl.dt.xform;
   pp.shift           = 0;
-  pp.pivot           = pivot;
+  pp.pivot           = sp.prefix;
   launch_downsweep<KeyT, PAY, true>(L, pl, K_SPLIT, true, true, pp);
+}
+
+// misort_select: the selection, one more read of the row for the neighbours of the kth key,
+// and the values written out
+template <typename KeyT>
+static void select_rows(Launcher& L, const PartLayout& u, const void* vin, long long kth, void* kth_out,
+                        void* next_out, void* max_out, char* S)
+{
+  const Plan& pl              = u.pl;
+  const SelectParams<KeyT> sp = run_selection<KeyT>(L, u, vin, kth, S, true);
+  if (next_out)
+    L.run(K_SELECT_NEIGHBOURS, [&] {
+      hipLaunchKernelGGL((select_above_kernel<KeyT, true>), dim3((unsigned)pl.n_chunks), dim3(SEL_NT), 0,
+                         L.stream, sp);
+      hipLaunchKernelGGL((select_above_kernel<KeyT, false>), dim3((unsigned)pl.n_chunks), dim3(SEL_NT), 0,
+                         L.stream, sp);
+    });
+  L.run(K_SELECT_EMIT, [&] {
+    hipLaunchKernelGGL((select_emit_kernel<KeyT>), dim3((unsigned)((pl.rows + 255) / 256)), dim3(256), 0,
+                       L.stream, sp, (uint32_t)pl.rows, reinterpret_cast<KeyT*>(kth_out),
+                       reinterpret_cast<KeyT*>(next_out), reinterpret_cast<KeyT*>(max_out));
+  });
 }
 
 template <typename KeyT>
@@ -1452,6 +1495,58 @@ int misort_partition(int dtype, const void* values_in, void* values_out, int64_t
   } else if (!want_indices && inplace) {
     launch_copy(L, K_COPY, values_out, S + u.off_stage, volume * eb);
   }
+  if (L.err != hipSuccess)
+    return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
+  return MISORT_OK;
+}
+
+// does misort_select serve this case?  (rows long enough for the radix path, 4- and 8-byte
+// real element types, kth inside the row)
+static bool select_served(const PartLayout& u) { return u.select && u.pl.dt.bytes >= 4 && u.pl.dt.xform != XF_COMPLEX; }
+
+size_t misort_select_scratch_bytes(int dtype, size_t volume, size_t sort_dim_size, long long kth)
+{
+  PartLayout u;
+  if (volume == 0) return 0;
+  if (partition_layout(dtype, volume, sort_dim_size, false, kth, u, true) != MISORT_OK) return 0;
+  return select_served(u) ? u.total : 0;
+}
+
+int misort_select(int dtype, const void* values_in, size_t volume, size_t sort_dim_size, long long kth,
+                  void* kth_out, void* next_out, void* max_out, void* scratch, size_t scratch_bytes,
+                  void* stream)
+{
+  if (volume == 0) return MISORT_OK;
+  Launcher L;
+  L.stream = reinterpret_cast<hipStream_t>(stream);
+  PartLayout u;
+  int rc = partition_layout(dtype, volume, sort_dim_size, false, kth, u, true);
+  if (rc != MISORT_OK) return rc;
+  if (!select_served(u))
+    return fail(MISORT_ERR_UNSUPPORTED,
+                "select: serves 4- and 8-byte real element types, rows long enough for the radix "
+                "path and kth inside the row; sort instead");
+  if (next_out && (unsigned long long)kth + 1 >= u.pl.row_len)
+    return fail(MISORT_ERR_UNSUPPORTED, "select: no element follows kth in the row");
+  if (!values_in || !scratch || (!kth_out && !next_out && !max_out))
+    return fail(MISORT_ERR_NULL, "select: NULL pointer");
+  if (scratch_bytes < u.total) return fail(MISORT_ERR_SCRATCH, "select: scratch too small");
+  const size_t eb = u.pl.dt.bytes;
+  auto misaligned = [](const void* p, size_t a) { return p && (reinterpret_cast<uintptr_t>(p) % a) != 0; };
+  if (misaligned(values_in, eb) || misaligned(kth_out, eb) || misaligned(next_out, eb) ||
+      misaligned(max_out, eb) || misaligned(scratch, 256))
+    return fail(MISORT_ERR_ALIGN, "select: misaligned pointer");
+  char* S = reinterpret_cast<char*>(scratch);
+  auto overlaps = [&](const void* p, size_t bytes) {
+    if (!p) return false;
+    const char* b = reinterpret_cast<const char*>(p);
+    return b < S + u.total && S < b + bytes;
+  };
+  if (overlaps(values_in, volume * eb) || overlaps(kth_out, u.pl.rows * eb) ||
+      overlaps(next_out, u.pl.rows * eb) || overlaps(max_out, u.pl.rows * eb))
+    return fail(MISORT_ERR_ALIAS, "scratch overlaps an input or output buffer");
+  if (eb == 4) select_rows<uint32_t>(L, u, values_in, kth, kth_out, next_out, max_out, S);
+  else select_rows<uint64_t>(L, u, values_in, kth, kth_out, next_out, max_out, S);
   if (L.err != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
   return MISORT_OK;

@@ -73,6 +73,8 @@ struct SelectParams {
   uint32_t* cand_chunk;           // the chunk each candidate came from
   unsigned long long* cand_n;     // per row: candidates written
   uint64_t cand_cap;
+  unsigned long long* n_equal;    // per row: keys equal to the kth key (known after the last pick)
+  unsigned long long* above_max;  // per row: smallest key above the kth key, largest key (misort_select only)
   uint32_t* cand_less_eq;         // per chunk: candidates below the kth key, and equal to it
   // outputs for the split pass (what its own counting pass would have written)
   uint32_t* chunk_hist;           // [chunk][RADIX]: keys below / equal / above in 0 / 1 / 2
@@ -125,6 +127,7 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
   // (one instance of the loop per state, so that the plain pass carries none of the rest)
   auto scan = [&](auto state_tag) {
     constexpr uint32_t ST = decltype(state_tag)::value;
+    KeyT top{};                 // the largest key seen (wanted of pass 0 by misort_select)
     uint32_t n_buf        = 0;  // APPEND: keys in this wavefront's part of cbuf (same in every lane)
     KeyT* wbuf            = cbuf + wave * CB;
     auto flush = [&] {
@@ -142,6 +145,7 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
       const KeyT k     = ST == SEL_CAND ? raw : KeyOps<KeyT>::to_key(raw, p.xform);
       const bool match = valid && select_matches(k, pre, shift);
       if (match) atomicAdd(&my[KeyOps<KeyT>::digit(k, shift) * COPIES], 1u);
+      if constexpr (ST == SEL_ROW && sizeof(KeyT) <= 8) top = key_lt(top, k) ? k : top;
       if constexpr (ST == SEL_APPEND) {
         const uint64_t m = __ballot(match);
         if (m) {
@@ -174,6 +178,18 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
       if (n_buf) flush();
     } else {
       for (uint64_t i = i0 + threadIdx.x; i < b1; i += SEL_NT) count(base[i], true);
+    }
+    if constexpr (ST == SEL_ROW && sizeof(KeyT) <= 8) {
+      if (p.above_max && pass == 0) {  // (every row is in this state in pass 0)
+        unsigned long long hi = 0;
+        if constexpr (sizeof(KeyT) <= 8) hi = top;
+#pragma unroll
+        for (int s = 32; s > 0; s >>= 1) {
+          const unsigned long long h2 = __shfl_xor(hi, s, 64);
+          hi = h2 > hi ? h2 : hi;
+        }
+        if (lane == 0 && b1 > b0) atomicMax(&p.above_max[2 * (uint64_t)row + 1], hi);
+      }
     }
   };
   if (st == SEL_ROW) scan(std::integral_constant<uint32_t, SEL_ROW>{});
@@ -213,8 +229,9 @@ __global__ void __launch_bounds__(RADIX) select_pick_kernel(SelectParams<KeyT> p
   unsigned long long before = incl - c;
   for (int w = 0; w < wave; ++w) before += wave_tot[w];
   if (c != 0 && before <= k && k < before + c) {  // exactly one thread
-    p.prefix[row] = select_with_byte(p.prefix[row], (uint32_t)d, shift);
-    p.kleft[row]  = k - before;
+    p.prefix[row]  = select_with_byte(p.prefix[row], (uint32_t)d, shift);
+    p.kleft[row]   = k - before;
+    p.n_equal[row] = c;  // (what the last pass leaves here is the count of the whole key)
     const uint32_t st = p.state[row];
     if (st == SEL_APPEND) {
       p.state[row]     = SEL_CAND;
@@ -235,6 +252,10 @@ __global__ void __launch_bounds__(256) select_init_kernel(SelectParams<KeyT> p, 
     p.state[r]     = SEL_ROW;
     p.cand_from[r] = p.n_passes;
     p.cand_n[r]    = 0;
+    if (p.above_max) {
+      p.above_max[2 * (uint64_t)r]     = ~0ull;
+      p.above_max[2 * (uint64_t)r + 1] = 0;
+    }
   }
 }
 
@@ -329,6 +350,94 @@ __global__ void __launch_bounds__(RADIX) select_chunk_counts_kernel(SelectParams
   if (c)
     atomicAdd(&p.slab_tot[((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX + d],
               (unsigned long long)c);
+}
+
+// grid: n_chunks, after the last pick; keys of at most 8 bytes.  For callers that want the
+// key after the kth one instead of a partitioned row: the smallest key above the kth key,
+// into above_max[2 * row] (all ones on entry).  Run twice: with CAND over the candidates of
+// the rows that have some (the key is nearly always among them), then without over the rows
+// themselves, where the workgroups of a row leave at once unless the answer is still open:
+// as many keys equal the kth key as lie at or before kth, and the candidates had nothing
+// above it.  (The largest key of the row, the other word, comes from the first histogram pass.)
+template <typename KeyT, bool CAND>
+__global__ void __launch_bounds__(SEL_NT) select_above_kernel(SelectParams<KeyT> p)
+{
+  static_assert(sizeof(KeyT) <= 8, "keys of at most 8 bytes");
+  __shared__ unsigned long long wmin[SEL_NT / 64];
+  const uint32_t row = blockIdx.x / p.chunks_per_row, chunk = blockIdx.x % p.chunks_per_row;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (p.kleft[row] + 1 < p.n_equal[row]) return;  // the key at kth + 1 equals the kth key
+  const KeyT kth = p.prefix[row];
+  const KeyT* base;
+  uint64_t b0, b1;
+  if constexpr (CAND) {
+    if (p.cand_from[row] >= p.n_passes) return;
+    const uint64_t n_c = p.cand_n[row];
+    const uint64_t per = (n_c + p.chunks_per_row - 1) / p.chunks_per_row;
+    base = p.cand + (uint64_t)row * p.cand_cap;
+    b0   = (uint64_t)chunk * per;
+    b1   = b0 + per < n_c ? b0 + per : n_c;
+  } else {
+    // (plain loads of a word that atomics of the launch before wrote: that launch is complete)
+    if (p.above_max[2 * (uint64_t)row] != ~0ull) return;
+    base = p.in + (uint64_t)row * p.row_len;
+    b0   = (uint64_t)chunk * p.chunk_len;
+    b1   = b0 + p.chunk_len;
+    if (b1 > p.row_len) b1 = p.row_len;
+  }
+  if (b0 >= b1) return;
+  KeyT above = (KeyT)~(KeyT)0;
+  auto look = [&](KeyT raw) {
+    const KeyT k = CAND ? raw : KeyOps<KeyT>::to_key(raw, p.xform);
+    above        = (k > kth && k < above) ? k : above;
+  };
+  constexpr int V = 16 / sizeof(KeyT);
+  struct alignas(16) Vec {
+    KeyT v[V];
+  };
+  uint64_t i0 = b0;
+  if ((reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
+    const uint64_t nvec = (b1 - b0) / V;
+    stream_vectors<4>(reinterpret_cast<const Vec*>(base + b0), nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) look(r.v[e]);
+    });
+    i0 = b0 + nvec * V;
+  }
+  for (uint64_t i = i0 + threadIdx.x; i < b1; i += SEL_NT) look(base[i]);
+  // (a key above the kth key that is all ones leaves the word as it is: all ones)
+  unsigned long long lo = above;
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) {
+    const unsigned long long l2 = __shfl_xor(lo, s, 64);
+    lo = l2 < lo ? l2 : lo;
+  }
+  if (lane == 0) wmin[wave] = lo;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SEL_NT / 64; ++w) lo = wmin[w] < lo ? wmin[w] : lo;
+    if (lo != ~0ull) atomicMin(&p.above_max[2 * (uint64_t)row], lo);
+  }
+}
+
+// grid-stride over rows, after the select_above_kernel launches: the kth key, the key at kth + 1
+// (the kth key again while more keys equal it than lie at or before kth, else the smallest
+// key above it) and the largest key, as values of the element type.  Floating-point values
+// come back in the form the keys keep: zeros as +0, every NaN as the default NaN.
+template <typename KeyT>
+__global__ void __launch_bounds__(256)
+select_emit_kernel(SelectParams<KeyT> p, uint32_t rows, KeyT* __restrict__ kth_out, KeyT* __restrict__ next_out,
+                   KeyT* __restrict__ max_out)
+{
+  for (uint32_t r = blockIdx.x * 256 + threadIdx.x; r < rows; r += gridDim.x * 256) {
+    const KeyT kth  = p.prefix[r];
+    const KeyT top  = (KeyT)p.above_max[2 * (uint64_t)r + 1];
+    KeyT above      = (KeyT)p.above_max[2 * (uint64_t)r];
+    if (above > top) above = top;  // nothing above: the row ends at kth (callers do not ask then)
+    if (kth_out) kth_out[r] = KeyOps<KeyT>::from_key(kth, p.xform);
+    if (next_out) next_out[r] = KeyOps<KeyT>::from_key(p.kleft[r] + 1 < p.n_equal[r] ? kth : above, p.xform);
+    if (max_out) max_out[r] = KeyOps<KeyT>::from_key(top, p.xform);
+  }
 }
 
 }  // namespace misort

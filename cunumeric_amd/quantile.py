@@ -110,37 +110,58 @@ def _from_torch(t: torch.Tensor, dtype) -> ndarray:
     return ndarray(tuple(t.shape), dtype, _buf=t.reshape(-1).view(torch.uint8))
 
 
-def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool) -> dict[int, torch.Tensor]:
+def _select_rows(a: ndarray, k: int, want_next: bool):
+    """The elements at sorted positions k (and k + 1) of every row of ``a`` and the rows' last
+    element in sort order, by the library's selection (no row is moved); ``None`` where the
+    library does not serve the case."""
+    from . import _lib
+    from .config import to_core_dtype
+    from .runtime import runtime
+
+    lib = _lib.load()
+    code = to_core_dtype(a.dtype)
+    n = a.shape[-1]
+    need = lib.misort_select_scratch_bytes(code, a.size, n, k)
+    if not need:
+        return None
+    rows = a.size // n
+    scratch = runtime.alloc_bytes(need)
+    outs = [ndarray((rows,), a.dtype) for _ in range(3 if want_next else 2)]
+    kth, top = outs[0], outs[-1]
+    _lib.check(lib.misort_select(code, a._ptr(), a.size, n, k, kth._ptr(), outs[1]._ptr() if want_next else None,
+                                 top._ptr(), scratch.data_ptr(), need, runtime.stream_handle()))
+    shape = tuple(a.shape[:-1])
+    return [o.to_torch().reshape(shape) for o in outs]
+
+
+def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool):
     """``a`` has the reduction axis last: the samples at the sorted positions ``wanted`` of
-    every row, as tensors of the row shape.  One or two adjacent positions on long rows are
-    found by selection (partition around the lower one; the upper one is then the smallest
-    element behind it); anything else sorts the rows."""
-    from .module import partition, sort
+    every row, as tensors of the row shape, and (or None) which rows hold a NaN.  One or two
+    adjacent positions on long rows are found by selection: two or three reads of the rows
+    instead of a sort, and the rows' largest element, which comes with it, tells the NaNs.
+    Anything else sorts the rows."""
+    from .module import sort
 
     n = a.shape[-1]
     wanted = sorted(set(wanted))
-    # (signed integers and floats: the reduction that picks the upper neighbour is a torch op)
-    select = (len(wanted) <= 2 and wanted[-1] - wanted[0] <= 1 and n >= (1 << 16) and
-              a.dtype.itemsize >= 4 and a.dtype.kind in "fi")
-    if select:
+    if (len(wanted) <= 2 and wanted[-1] - wanted[0] <= 1 and n >= (1 << 16) and a.dtype.itemsize >= 4 and
+            a.dtype.kind in "fiu" and a.size):
         k = wanted[0]
-        if overwrite_input:
-            a.partition(k, axis=-1)
-            part = a
-        else:
-            part = partition(a, k, axis=-1)
-        t = part.to_torch()
-        out = {k: t[..., k]}
-        if len(wanted) == 2:
-            out[k + 1] = t[..., k + 1:].amin(dim=-1)
-        return out
+        found = _select_rows(a, k, len(wanted) == 2)
+        if found is not None:
+            out = {k: found[0]}
+            if len(wanted) == 2:
+                out[k + 1] = found[1]
+            return out, (torch.isnan(found[-1]) if a.dtype.kind == "f" else None)
     if overwrite_input:
         a.sort(axis=-1)
         s = a
     else:
         s = sort(a, axis=-1)
     t = s.to_torch()
-    return {k: t[..., k] for k in wanted}
+    # (NaNs sort last)
+    has_nan = torch.isnan(t[..., -1]) if a.dtype.kind == "f" and n else None
+    return {k: t[..., k] for k in wanted}, has_nan
 
 
 def _reduction_rows(a: ndarray, axis):
@@ -202,7 +223,7 @@ def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: 
     # ---- the samples around every quantile ---------------------------------------------
     places = [_position(method, float(qv), n) for qv in q_arr.reshape(-1)]
     wanted = [p[0] for p in places] + [p[1] for p in places]
-    stats = _order_statistics(rows, wanted, overwrite_input)
+    stats, has_nan = _order_statistics(rows, wanted, overwrite_input)
     to_dtype = a.dtype if method in _SAMPLE_METHODS else np.dtype(np.float64)
     tdt = _torch_dtype(to_dtype)
     results = []
@@ -217,12 +238,10 @@ def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: 
         results.append(r)
     res = torch.stack(results, dim=0) if results else torch.empty((0, *kept_shape), dtype=tdt,
                                                                   device=rows.to_torch().device)
-    if a.dtype.kind == "f":
-        # a sample with a NaN has no quantiles: its largest element (NaNs sort last) tells
-        has_nan = torch.isnan(rows.to_torch()).any(dim=-1) if rows.size else None
-        if has_nan is not None and bool(has_nan.any()):
-            nan = torch.tensor(float("nan"), dtype=tdt, device=res.device)
-            res = torch.where(has_nan.unsqueeze(0), nan, res)
+    if has_nan is not None and results:
+        # a sample with a NaN has no quantiles: its last element in sort order tells
+        nan = torch.tensor(float("nan"), dtype=tdt, device=res.device)
+        res = torch.where(has_nan.unsqueeze(0), nan, res)
     if keepdims:
         remaining = tuple(1 if k in axes else original_shape[k] for k in range(nd))
     else:

@@ -193,6 +193,27 @@ int misort_partition(int dtype, const void* values_in, void* values_out, int64_t
                      void* scratch, size_t scratch_bytes, void* stream);
 
 /*
+ * The selection alone, for callers that want order statistics and not a partitioned row
+ * (quantile / percentile: cunumeric/module.py:8248-8531 sorts the whole array and reads
+ * two elements per quantile; src/cunumeric/sort/sort.cu:52-85 is that sort).  Per row of
+ * sort_dim_size elements: kth_out[row] = the element a sort would leave at position kth,
+ * next_out[row] = the one at kth + 1 (kth + 1 must lie inside the row), max_out[row] = the
+ * last element in sort order (NaN for a floating-point row that holds a NaN).  Each of the
+ * three may be NULL; each has volume / sort_dim_size elements of the element type.  The row
+ * is read, not written.  Floating-point results come back as the keys keep them: a zero as
+ * +0, a NaN as the default quiet NaN.  Served: 4- and 8-byte integer and floating-point
+ * types on rows long enough for the radix path with 0 <= kth < sort_dim_size; otherwise
+ * misort_select_scratch_bytes returns 0 and misort_select MISORT_ERR_UNSUPPORTED (sort
+ * instead).  Work: one read of the row per leading key byte until the keys that still match
+ * are few (two reads when the leading bytes vary), and one more for next_out only when those
+ * keys hold nothing above the kth key; against four to eight scattered passes of a sort.
+ */
+size_t misort_select_scratch_bytes(int dtype, size_t volume, size_t sort_dim_size, long long kth);
+int misort_select(int dtype, const void* values_in, size_t volume, size_t sort_dim_size, long long kth,
+                  void* kth_out, void* next_out, void* max_out, void* scratch, size_t scratch_bytes,
+                  void* stream);
+
+/*
  * Sort a dense (outer, k, inner) array along its middle axis: every column (o, :, i) on its
  * own, result in the same layout; give values_out (may be values_in) or indices_out
  * (positions along the axis + index_offset), not both.  Served for short axes (k up to

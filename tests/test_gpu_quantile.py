@@ -131,14 +131,16 @@ def test_output_dtype_rule_and_errors():
         num.percentile(arr, 101)
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64, np.uint32, np.uint64])
 @pytest.mark.parametrize("method", ("linear", "hazen", "lower", "nearest", "averaged_inverted_cdf"))
 def test_long_rows_take_the_selection_path(dtype, method):
-    """One quantile of long rows: found by radix select + one split pass, not a sort."""
+    """One quantile of long rows: found by radix select (no row is sorted or moved)."""
     rng = np.random.default_rng(23)
     n = (1 << 17) + 77
     if np.dtype(dtype).kind == "f":
         a = rng.standard_normal((3, n)).astype(dtype)
+    elif np.dtype(dtype).kind == "u":
+        a = rng.integers(0, 2000, (3, n)).astype(dtype)
     else:
         a = rng.integers(-1000, 1000, (3, n)).astype(dtype)
     a64 = a.astype(np.float64) if np.dtype(dtype) == np.float32 else a  # NumPy blends in the input's precision
@@ -160,3 +162,9 @@ def test_rows_with_nan_have_no_quantile():
     for method in ("linear", "lower", "midpoint"):
         check(num.quantile(a, [0.1, 0.9], axis=1, method=method),
               np.quantile(a, [0.1, 0.9], axis=1, method=method), method)
+    # long rows (the selection path): the largest element of a row tells the NaN
+    b = np.random.default_rng(4).standard_normal((3, 70001))
+    b[2, 5] = np.nan
+    for method in ("linear", "lower", "midpoint"):
+        for q in (0.5, 0.999):
+            check(num.quantile(b, q, axis=1, method=method), np.quantile(b, q, axis=1, method=method), method)
