@@ -449,7 +449,7 @@ constexpr bool is_float_width()
 }
 
 // the scatter kernel of one pass
-template <typename KeyT, int PAY, bool PART>
+template <typename KeyT, int PAY>
 static void launch_downsweep(Launcher& L, const Plan& pl, int id, bool first, bool last,
                              const PassParams& pp)
 {
@@ -459,21 +459,18 @@ static void launch_downsweep(Launcher& L, const Plan& pl, int id, bool first, bo
   constexpr int OCC = TileCfg<sizeof(KeyT), PAY>::OCC;
   constexpr int G   = TileCfg<sizeof(KeyT), PAY>::G;
   L.run(id, [&] {
-    if constexpr (!PART && PAY == PAY_NONE && sizeof(KeyT) == 8) {
+    if constexpr (PAY == PAY_NONE && sizeof(KeyT) == 8) {
       if (pp.digits_out) {  // keys-only pass that also writes the digit side-band
         if (first)
-          hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, false, NT, IPT, G, OCC, false, true>), grid,
+          hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, false, NT, IPT, G, OCC, true>), grid,
                              dim3(NT), 0, L.stream, pp);
         else
-          hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, false, false, NT, IPT, G, OCC, false, true>), grid,
+          hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, false, false, NT, IPT, G, OCC, true>), grid,
                              dim3(NT), 0, L.stream, pp);
         return;
       }
     }
-    if constexpr (PART)
-      hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, true, NT, IPT, G, OCC, true>), grid, dim3(NT),
-                         0, L.stream, pp);
-    else if (first && last)
+    if (first && last)
       hipLaunchKernelGGL((downsweep_kernel<KeyT, PAY, true, true, NT, IPT, G, OCC>), grid, dim3(NT), 0,
                          L.stream, pp);
     else if (first)
@@ -514,7 +511,7 @@ static void launch_pass(Launcher& L, const Plan& pl, bool first, bool last, cons
   });
 
   const int id = first ? (last ? K_DOWN_ONLY : K_DOWN_FIRST) : (last ? K_DOWN_LAST : K_DOWN_MIDDLE);
-  launch_downsweep<KeyT, PAY, false>(L, pl, id, first, last, pp);
+  launch_downsweep<KeyT, PAY>(L, pl, id, first, last, pp);
 }
 
 static void launch_zero(Launcher& L, void* p, size_t bytes)
@@ -774,13 +771,12 @@ static void count8_sort(Launcher& L, const Plan& pl, const SortArgs& a)
 struct PartLayout {
   Plan pl;              // geometry of the split pass (and the plan of the fallback sort)
   bool select = false;  // false: the ordinary sort is used (it is a valid partition)
-  bool by_index = false;  // values wanted but the key is not invertible: split positions, gather
-  size_t off_pivot = 0, off_kleft = 0, off_ghist = 0, off_stage = 0, off_idx = 0, off_src = 0;
+  size_t off_pivot = 0, off_kleft = 0, off_ghist = 0, off_stage = 0;
   // radix select: per-row state and candidate counts, the candidate keys of every row with
   // the chunks they came from, what every chunk counted in every pass
   size_t off_sel_state = 0, off_cand_from = 0, off_cand_n = 0, off_cand = 0, off_cand_chunk = 0, cand_cap = 0;
   size_t off_cand_less_eq = 0, off_pass_hist = 0, zeroed_end = 0;
-  size_t off_n_equal = 0, off_above_max = 0;
+  size_t off_n_equal = 0, off_above_max = 0, off_chunk_cls = 0, off_chunk_off = 0;
   size_t total = 0;
 };
 
@@ -790,9 +786,7 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
 {
   DtypeInfo dt;
   if (!dtype_info(dtype, dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
-  const bool lossy = dt.xform == XF_FLOAT || dt.xform == XF_COMPLEX;  // key does not keep all bits
-  u.by_index       = !want_indices && lossy && !select_only;
-  int rc = make_plan(dtype, volume, sort_dim_size, want_indices || u.by_index, false, u.pl);
+  int rc = make_plan(dtype, volume, sort_dim_size, want_indices, false, u.pl);
   if (rc != MISORT_OK) return rc;
   // 1- and 2-byte values are counted, which beats selecting; their positions are selected
   u.select = u.pl.strategy == S_RADIX && u.pl.pay != PAY_I64 && kth >= 0 &&
@@ -816,11 +810,10 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   u.off_pivot       = take(pl.rows * 16);
   u.off_kleft       = take(pl.rows * sizeof(unsigned long long));
   u.off_ghist       = take(pl.rows * RADIX * sizeof(unsigned long long));
-  pl.slab_tot_bytes = pl.rows * pl.slabs_per_row * RADIX * sizeof(unsigned long long);
-  pl.off_slab_tot   = take(pl.slab_tot_bytes);  // cleared together with the counters before it
-  u.off_cand_less_eq = take(pl.n_chunks * 2 * sizeof(uint32_t));  // and with those after it
+  u.off_cand_less_eq = take(pl.n_chunks * 2 * sizeof(uint32_t));  // cleared together with the counters before it
   u.zeroed_end      = off;
-  pl.off_chunk_hist = take(pl.n_chunks * RADIX * sizeof(uint32_t));
+  u.off_chunk_cls   = take(pl.n_chunks * 4 * sizeof(uint32_t));
+  u.off_chunk_off   = take(pl.n_chunks * 4 * sizeof(unsigned long long));
   u.off_pass_hist   = take((size_t)dt.bytes * pl.n_chunks * RADIX * sizeof(uint32_t));
   u.off_sel_state   = take(pl.rows * sizeof(uint32_t));
   u.off_n_equal     = take(pl.rows * sizeof(unsigned long long));
@@ -830,11 +823,7 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   u.cand_cap        = pl.row_len / 8 + 1;  // keys that still match, once they are this few
   u.off_cand        = take(pl.rows * u.cand_cap * pl.dt.bytes);
   u.off_cand_chunk  = take(pl.rows * u.cand_cap * sizeof(uint32_t));
-  if (!select_only) {
-    u.off_stage = take(pl.volume * pl.dt.bytes);      // values when in == out
-    u.off_idx   = take(pl.volume * sizeof(int64_t));  // positions when values are gathered
-    u.off_src   = take(pl.volume * pl.dt.bytes);      // copy of the input for an in-place gather
-  }
+  if (!select_only && !want_indices) u.off_stage = take(pl.volume * pl.dt.bytes);  // values when in == out
   u.total = off;
   return MISORT_OK;
 }
@@ -867,10 +856,8 @@ static SelectParams<KeyT> run_selection(Launcher& L, const PartLayout& u, const 
   sp.n_equal         = reinterpret_cast<unsigned long long*>(S + u.off_n_equal);
   sp.above_max       = neighbours ? reinterpret_cast<unsigned long long*>(S + u.off_above_max) : nullptr;
   sp.cand_less_eq    = reinterpret_cast<uint32_t*>(S + u.off_cand_less_eq);
-  sp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
-  sp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
-  sp.chunks_per_slab = (uint32_t)pl.chunks_per_slab;
-  sp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
+  sp.chunk_cls       = reinterpret_cast<uint32_t*>(S + u.off_chunk_cls);
+  sp.chunk_off       = reinterpret_cast<unsigned long long*>(S + u.off_chunk_off);
   const dim3 grid((unsigned)pl.n_chunks);
   const dim3 rgrid((unsigned)pl.rows);
 
@@ -891,39 +878,32 @@ static SelectParams<KeyT> run_selection(Launcher& L, const PartLayout& u, const 
   return sp;
 }
 
-template <typename KeyT, int PAY>
-static void partition_select_rows(Launcher& L, const PartLayout& u, const void* vin, void* keys_out,
-                                  void* pay_out, long long kth, int64_t index_offset, char* S)
+// partition / argpartition: the selection, then the split around the key it found.  Give
+// values_out (which receives the values as they came in) or pos_out.
+template <typename KeyT>
+static void partition_select_rows(Launcher& L, const PartLayout& u, const void* vin, void* values_out,
+                                  int64_t* pos_out, long long kth, int64_t index_offset, char* S)
 {
   const Plan& pl              = u.pl;
   const SelectParams<KeyT> sp = run_selection<KeyT>(L, u, vin, kth, S, false);
   const dim3 grid((unsigned)pl.n_chunks);
-  // the counts the split pass needs, from what the passes above counted per chunk
+  // where the split puts the keys of every chunk, from what the passes above counted per chunk
   L.run(K_SELECT_COUNTS, [&] {
     hipLaunchKernelGGL((select_cand_counts_kernel<KeyT>), grid, dim3(SEL_NT), 0, L.stream, sp);
     hipLaunchKernelGGL((select_chunk_counts_kernel<KeyT>), grid, dim3(RADIX), 0, L.stream, sp);
+    hipLaunchKernelGGL((select_chunk_offsets_kernel<KeyT>), dim3((unsigned)pl.rows), dim3(256), 0, L.stream, sp);
   });
-
-  PassParams pp{};
-  pp.keys_in         = vin;
-  pp.keys_out        = keys_out;
-  pp.pay_in          = nullptr;
-  pp.pay_out         = pay_out;
-  pp.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_chunk_hist);
-  pp.slab_tot        = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot);
-  pp.slab_tot_next   = nullptr;
-  pp.row_len         = pl.row_len;
-  pp.index_offset    = index_offset;
-  pp.tile            = (uint32_t)pl.tile;
-  pp.tiles_per_row   = (uint32_t)pl.tiles_per_row;
-  pp.tiles_per_chunk = (uint32_t)pl.tiles_per_chunk;
-  pp.chunks_per_row  = (uint32_t)pl.chunks_per_row;
-  pp.chunks_per_slab = (uint32_t)pl.chunks_per_slab;
-  pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
-  pp.xform           = pl.dt.xform;
-  pp.shift           = 0;
-  pp.pivot           = sp.prefix;
-  launch_downsweep<KeyT, PAY, true>(L, pl, K_SPLIT, true, true, pp);
+  constexpr int NT = 1024, IPT = sizeof(KeyT) >= 16 ? 4 : 8;
+  L.run(K_SPLIT, [&] {
+    if (pos_out) {
+      hipLaunchKernelGGL((select_split_kernel<KeyT, true, NT, IPT>), grid, dim3(NT), 0, L.stream, sp, nullptr,
+                         pos_out, index_offset);
+    } else {
+      if constexpr (sizeof(KeyT) > 2)  // (values of 1 and 2 bytes are counted, not selected)
+        hipLaunchKernelGGL((select_split_kernel<KeyT, false, NT, IPT>), grid, dim3(NT), 0, L.stream, sp,
+                           reinterpret_cast<KeyT*>(values_out), nullptr, index_offset);
+    }
+  });
 }
 
 // misort_select: the selection, one more read of the row for the neighbours of the kth key,
@@ -946,16 +926,6 @@ static void select_rows(Launcher& L, const PartLayout& u, const void* vin, long 
                        L.stream, sp, (uint32_t)pl.rows, reinterpret_cast<KeyT*>(kth_out),
                        reinterpret_cast<KeyT*>(next_out), reinterpret_cast<KeyT*>(max_out));
   });
-}
-
-template <typename KeyT>
-static void partition_select_pay(Launcher& L, const PartLayout& u, const void* vin, void* keys_out,
-                                 void* pay_out, long long kth, int64_t index_offset, char* S)
-{
-  if (u.pl.pay == PAY_NONE)
-    partition_select_rows<KeyT, PAY_NONE>(L, u, vin, keys_out, pay_out, kth, index_offset, S);
-  else
-    partition_select_rows<KeyT, PAY_IDX32>(L, u, vin, keys_out, pay_out, kth, index_offset, S);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1464,18 +1434,8 @@ int misort_partition(int dtype, const void* values_in, void* values_out, int64_t
       return fail(MISORT_ERR_ALIAS, "scratch overlaps an input or output buffer");
   }
   const bool inplace = values_out == values_in;
-  void* keys_out     = nullptr;
-  void* pay_out      = nullptr;
-  if (want_indices) {
-    pay_out = indices_out;
-  } else if (u.by_index) {
-    pay_out = S + u.off_idx;
-  } else {
-    keys_out = inplace ? static_cast<void*>(S + u.off_stage) : values_out;
-  }
-  // positions travel relative to the row; the offset is added when they leave the library
-  const int64_t off = want_indices ? index_offset : 0;
-#define MISORT_PART_CASE(KEY) partition_select_pay<KEY>(L, u, values_in, keys_out, pay_out, kth, off, S)
+  void* vals         = want_indices ? nullptr : (inplace ? static_cast<void*>(S + u.off_stage) : values_out);
+#define MISORT_PART_CASE(KEY) partition_select_rows<KEY>(L, u, values_in, vals, indices_out, kth, index_offset, S)
   switch (eb) {
     case 1: MISORT_PART_CASE(uint8_t); break;
     case 2: MISORT_PART_CASE(uint16_t); break;
@@ -1484,17 +1444,7 @@ int misort_partition(int dtype, const void* values_in, void* values_out, int64_t
     default: MISORT_PART_CASE(u128); break;
   }
 #undef MISORT_PART_CASE
-  if (u.by_index) {
-    const void* src = values_in;
-    if (inplace) {
-      launch_copy(L, K_COPY, S + u.off_src, values_in, volume * eb);
-      src = S + u.off_src;
-    }
-    launch_gather(L, K_GATHER, eb, src, values_out, reinterpret_cast<const int64_t*>(S + u.off_idx),
-                  u.pl.rows, u.pl.row_len, 0);
-  } else if (!want_indices && inplace) {
-    launch_copy(L, K_COPY, values_out, S + u.off_stage, volume * eb);
-  }
+  if (!want_indices && inplace) launch_copy(L, K_COPY, values_out, S + u.off_stage, volume * eb);
   if (L.err != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("HIP error: ") + hipGetErrorString(L.err));
   return MISORT_OK;

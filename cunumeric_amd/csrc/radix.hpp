@@ -37,19 +37,6 @@
 
 namespace misort {
 
-// Digit value of a key in one pass.  PART: the pass is a three-way split around a pivot
-// key instead of a radix digit: 0 below the pivot, 1 equal to it, 2 above (the single pass
-// that partition / argpartition run once the pivot is known).
-template <typename KeyT, bool PART>
-__device__ __forceinline__ uint32_t pass_digit(KeyT k, int shift, KeyT pivot)
-{
-  if constexpr (PART) {
-    return key_lt(k, pivot) ? 0u : (key_eq(k, pivot) ? 1u : 2u);
-  } else {
-    return KeyOps<KeyT>::digit(k, shift);
-  }
-}
-
 // ---------------------------------------------------------------------------------------
 // small utility kernels
 // ---------------------------------------------------------------------------------------
@@ -109,7 +96,6 @@ struct PassParams {
   int shift;
   int xform;
   int rank_by_add;    // downsweep: rank with returning LDS adds where the chunk's digits allow
-  const void* pivot;  // PART passes: one pivot key per row
 };
 
 // key_bits holds this many copies of its four words (their OR counts)
@@ -282,7 +268,7 @@ __global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
 // and a private LDS histogram.  SPECIALS (first pass of a keys-only float sort) also counts
 // zeros / NaNs per wave sub-chunk for the patch that restores their bit patterns.
 // ---------------------------------------------------------------------------------------
-template <typename KeyT, bool FIRST, bool SPECIALS, int NT, bool PART = false>
+template <typename KeyT, bool FIRST, bool SPECIALS, int NT>
 __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
 {
   constexpr int NW = NT / 64;
@@ -296,8 +282,8 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   const uint32_t row   = blockIdx.x / p.chunks_per_row;
   const uint32_t chunk = blockIdx.x % p.chunks_per_row;
   // (the counters are cleared while the words of the plan arrive)
-  for (int i = threadIdx.x; i < ((!FIRST && !PART && !SPECIALS) ? WORDS : NW * RADIX * COPIES); i += NT) lhist[i] = 0;
-  if constexpr (!FIRST && !PART) {
+  for (int i = threadIdx.x; i < ((!FIRST && !SPECIALS) ? WORDS : NW * RADIX * COPIES); i += NT) lhist[i] = 0;
+  if constexpr (!FIRST) {
     const PassPlan plan = plan_pass(p);
     if (plan.skip) return;  // every key has the same digit: the scatter of this pass is skipped too
     if (plan.const_digit >= 0) {
@@ -341,15 +327,13 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   const uint32_t first = SPLIT ? (uint32_t)lane : threadIdx.x;
   const uint32_t width = SPLIT ? 64u : (uint32_t)NT;
   uint32_t* my = lhist + wave * (RADIX * COPIES) + (lane & (COPIES - 1));
-  KeyT pivot{};
-  if constexpr (PART) pivot = reinterpret_cast<const KeyT*>(p.pivot)[row];
 
   uint32_t n_zero = 0, n_nan = 0, n_negzero = 0, n_neg = 0;
   // FIRST: OR of the keys and of their complements (which bits vary over the whole input)
   unsigned long long or_lo = 0, or_hi = 0, nor_lo = 0, nor_hi = 0;
   auto count = [&](KeyT raw) {
     const KeyT k = FIRST ? KeyOps<KeyT>::to_key(raw, p.xform) : raw;
-    if constexpr (FIRST && !PART) {
+    if constexpr (FIRST) {
       if constexpr (sizeof(KeyT) == 16) {
         or_lo |= k.lo;
         or_hi |= k.hi;
@@ -360,7 +344,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
         nor_lo |= (unsigned long long)(KeyT)~k;
       }
     }
-    atomicAdd(&my[pass_digit<KeyT, PART>(k, p.shift, pivot) * COPIES], 1u);
+    atomicAdd(&my[KeyOps<KeyT>::digit(k, p.shift) * COPIES], 1u);
     if constexpr (SPECIALS) {
       using F = FloatBits<KeyT>;
       const bool isn = float_is_nan(raw);
@@ -413,7 +397,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       if (n_neg) atomicAdd(&ctr[3], (unsigned long long)n_neg);
     }
   }
-  if constexpr (FIRST && !PART) {
+  if constexpr (FIRST) {
     if (p.key_bits_out) {
 #pragma unroll
       for (int s = 32; s > 0; s >>= 1) {
@@ -433,7 +417,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
     }
   }
   __syncthreads();
-  if constexpr (FIRST && !PART) {
+  if constexpr (FIRST) {
     // Atomics on one address queue up (about 10 ns each), so a workgroup adds its bits once,
     // to one of KEY_BITS_SLOTS copies of the words, and nobody waits for the result.
     if (p.key_bits_out && threadIdx.x < 4 && (sizeof(KeyT) == 16 || (threadIdx.x & 1) == 0)) {
@@ -507,10 +491,10 @@ __device__ __forceinline__ void load_tile_payload(const PassParams& p, uint64_t 
 // complete), and whenever the run passes a 128-byte boundary the waiting bytes and the new
 // ones up to that boundary go out together.
 template <typename KeyT, int PAY, bool FIRST, bool LAST, int NT, int IPT, int G, int OCC,
-          bool PART = false, bool SIDE = false>
+          bool SIDE = false>
 __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
 {
-  static_assert(!SIDE || (PAY == PAY_NONE && !LAST && !PART && (RADIX * G) / NT <= 8),
+  static_assert(!SIDE || (PAY == PAY_NONE && !LAST && (RADIX * G) / NT <= 8),
                 "the side-band is written by keys-only passes before the last");
   static_assert(NT % RADIX == 0 && (NT / 64) % (NT / RADIX) == 0, "whole groups of digit owners");
   static_assert((G & (G - 1)) == 0 && (RADIX * G) % NT == 0, "carry slots divide evenly");
@@ -555,11 +539,9 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   uint32_t tile_end       = tile0 + p.tiles_per_chunk;
   if (tile_end > p.tiles_per_row) tile_end = p.tiles_per_row;
   const uint64_t row_base = (uint64_t)row * p.row_len;
-  KeyT pivot{};
-  if constexpr (PART) pivot = reinterpret_cast<const KeyT*>(p.pivot)[row];
-  auto digit_of = [&](KeyT k) { return pass_digit<KeyT, PART>(k, p.shift, pivot); };
+  auto digit_of = [&](KeyT k) { return KeyOps<KeyT>::digit(k, p.shift); };
   int next_shift = p.shift + RADIX_BITS;  // digit position that the side-band carries
-  if constexpr (!PART && sizeof(KeyT) >= 4) {  // (shorter keys have no middle pass)
+  if constexpr (sizeof(KeyT) >= 4) {  // (shorter keys have no middle pass)
     const PassPlan plan = plan_pass(p);
     if (plan.skip) {
       // Every key of the input has the same digit here: the pass would copy every row onto
@@ -598,7 +580,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   // anyway, byte by byte next to the keys.  That costs a partly written 128-byte line per digit
   // value and tile, so it pays only where few digit values are in use (long runs per tile);
   // decided below from the row's counts, the same way by every workgroup of the row.
-  constexpr bool ADAPT = !SIDE && !PART && !LAST && sizeof(KeyT) >= 4 && (PAY != PAY_NONE || sizeof(KeyT) > 4);
+  constexpr bool ADAPT = !SIDE && !LAST && sizeof(KeyT) >= 4 && (PAY != PAY_NONE || sizeof(KeyT) > 4);
   bool side_on = false;
   KeyT* kout = reinterpret_cast<KeyT*>(p.keys_out);
   auto emit  = [&](unsigned long long dst, KeyT k, PayT v) {
@@ -713,7 +695,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
     if (tid < RADIX) run = row_base + base + incl - total + before;
     brun = run;
     // returning adds unless one digit value holds more than an eighth of the chunk
-    if (!PART && p.rank_by_add)
+    if (p.rank_by_add)
       rank_by_add = __builtin_amdgcn_readfirstlane((int)(mx * 8u <= tot)) != 0;
     __syncthreads();
   }

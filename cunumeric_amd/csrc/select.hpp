@@ -10,10 +10,10 @@
 // passes then read 1/256 of the data.  The state of a row (SEL_ROW / SEL_APPEND / SEL_CAND)
 // lives on the device and is advanced by select_pick_kernel.
 // After the last byte the pivot key is complete; partition / argpartition then run ONE
-// three-way split pass (the downsweep with PART) around it.  The counts that pass needs per
-// chunk (keys below / equal to / above the pivot) are put together from what the chunks
-// counted during the selection (select_cand_counts_kernel, select_chunk_counts_kernel), so
-// the row is not read once more to count them.  The reference
+// three-way split pass around it (select_split_kernel).  Where the keys of every chunk go
+// (those below / equal to / above the pivot) is put together from what the chunks counted
+// during the selection (select_cand_counts_kernel, select_chunk_counts_kernel,
+// select_chunk_offsets_kernel), so the row is not read once more to count them.  The reference
 // sorts completely for partition (cunumeric/deferred.py:3559-3578); NumPy only asks for
 // the element at kth to be in its sorted place with nothing larger before it and nothing
 // smaller after it.
@@ -27,7 +27,8 @@
 
 namespace misort {
 
-constexpr int SEL_NT = 256;
+constexpr int SEL_NT = 512;
+constexpr int SEL_U  = 8;  // 16-byte loads a lane keeps in flight in the histogram pass
 // where the histogram pass of a row reads its keys, and whether it writes candidates
 constexpr uint32_t SEL_ROW = 0, SEL_APPEND = 1, SEL_CAND = 2;
 
@@ -76,10 +77,9 @@ struct SelectParams {
   unsigned long long* n_equal;    // per row: keys equal to the kth key (known after the last pick)
   unsigned long long* above_max;  // per row: smallest key above the kth key, largest key (misort_select only)
   uint32_t* cand_less_eq;         // per chunk: candidates below the kth key, and equal to it
-  // outputs for the split pass (what its own counting pass would have written)
-  uint32_t* chunk_hist;           // [chunk][RADIX]: keys below / equal / above in 0 / 1 / 2
-  unsigned long long* slab_tot;   // [row][slab][RADIX], zero on entry
-  uint32_t chunks_per_slab, slabs_per_row;
+  // for the split pass
+  uint32_t* chunk_cls;            // [chunk][4]: keys below / equal to / above the kth key (and a pad)
+  unsigned long long* chunk_off;  // [chunk][4]: where the chunk's keys of each class go in the output
 };
 
 // grid: n_chunks.  Pass `pass` counts byte `shift / 8` of the keys that match the prefix.
@@ -151,21 +151,26 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
         if (m) {
           if (match) wbuf[n_buf + __popcll(m & ((1ull << lane) - 1))] = k;
           n_buf += __popcll(m);
-          if (n_buf > CB - 64) flush();
         }
       }
+    };
+    // (asked once per 16-byte load: V more keys per lane fit behind what is there)
+    auto flush_if_full = [&] {
+      if constexpr (ST == SEL_APPEND)
+        if (n_buf > CB - 64 * V) flush();
     };
     // 16-byte loads where the row allows it; in whole batches only when appending, so that the
     // rest is done with the wavefronts intact
     uint64_t i0 = b0;
     if (V > 1 && (reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
       uint64_t nvec = (b1 - b0) / V;
-      if (ST == SEL_APPEND) nvec -= nvec % ((uint64_t)SEL_NT * 4);
+      if (ST == SEL_APPEND) nvec -= nvec % ((uint64_t)SEL_NT * SEL_U);
       const Vec* vb = reinterpret_cast<const Vec*>(base + b0);
       if constexpr (sizeof(Vec) == 16) {
-        stream_vectors<4>(vb, nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
+        stream_vectors<SEL_U>(vb, nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
 #pragma unroll
           for (int e = 0; e < V; ++e) count(r.v[e], true);
+          flush_if_full();
         });
       }
       i0 = b0 + nvec * V;
@@ -174,6 +179,7 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
       for (uint64_t i = i0; i < b1; i += SEL_NT) {  // the same number of rounds for every lane
         const bool valid = i + threadIdx.x < b1;
         count(valid ? base[i + threadIdx.x] : KeyT{}, valid);
+        flush_if_full();
       }
       if (n_buf) flush();
     } else {
@@ -201,8 +207,8 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
     uint32_t c = 0;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const uint4 q = *reinterpret_cast<const uint4*>(&h[(w * RADIX + d) * COPIES]);
-      c += q.x + q.y + q.z + q.w;
+#pragma unroll
+      for (int e = 0; e < COPIES; ++e) c += h[(w * RADIX + d) * COPIES + e];
     }
     if (c) atomicAdd(&p.ghist[(uint64_t)row * RADIX + d], (unsigned long long)c);
     if (st != SEL_CAND) mine[d] = c;
@@ -345,11 +351,154 @@ __global__ void __launch_bounds__(RADIX) select_chunk_counts_kernel(SelectParams
   if (b1 > p.row_len) b1 = p.row_len;
   if (b0 > b1) b0 = b1;
   const uint32_t len = (uint32_t)(b1 - b0);
-  const uint32_t c   = d == 0 ? n_below : d == 1 ? n_equal : d == 2 ? len - n_below - n_equal : 0u;
-  p.chunk_hist[(uint64_t)blockIdx.x * RADIX + d] = c;
-  if (c)
-    atomicAdd(&p.slab_tot[((uint64_t)row * p.slabs_per_row + chunk / p.chunks_per_slab) * RADIX + d],
-              (unsigned long long)c);
+  if (d < 4) p.chunk_cls[4 * (uint64_t)blockIdx.x + d] = d == 0 ? n_below : d == 1 ? n_equal : d == 2 ? len - n_below - n_equal : 0u;
+}
+
+// grid: rows, 256 threads, after select_chunk_counts_kernel.  Where in the output the keys
+// of every chunk go: the row's keys below the kth key first, then those equal to it, then
+// those above, each class in the order of the chunks (so that equal keys keep their order).
+template <typename KeyT>
+__global__ void __launch_bounds__(256) select_chunk_offsets_kernel(SelectParams<KeyT> p)
+{
+  __shared__ unsigned long long wsum[3][4];
+  const uint32_t row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t* cls = p.chunk_cls + 4 * (uint64_t)row * p.chunks_per_row;
+  unsigned long long* off = p.chunk_off + 4 * (uint64_t)row * p.chunks_per_row;
+  // totals of the classes over the row
+  unsigned long long t[3] = {0, 0, 0};
+  for (uint32_t c = threadIdx.x; c < p.chunks_per_row; c += 256)
+    for (int k = 0; k < 3; ++k) t[k] += cls[4 * (uint64_t)c + k];
+  for (int k = 0; k < 3; ++k) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) t[k] += __shfl_xor(t[k], s, 64);
+    if (lane == 0) wsum[k][wave] = t[k];
+  }
+  __syncthreads();
+  unsigned long long carry[3];
+  const unsigned long long n_below = wsum[0][0] + wsum[0][1] + wsum[0][2] + wsum[0][3];
+  const unsigned long long n_equal = wsum[1][0] + wsum[1][1] + wsum[1][2] + wsum[1][3];
+  carry[0] = (unsigned long long)row * p.row_len;
+  carry[1] = carry[0] + n_below;
+  carry[2] = carry[1] + n_equal;
+  for (uint32_t c0 = 0; c0 < p.chunks_per_row; c0 += 256) {
+    const uint32_t c = c0 + threadIdx.x;
+    unsigned long long v[3], incl[3];
+    __syncthreads();  // wsum is free again
+    for (int k = 0; k < 3; ++k) {
+      v[k]    = c < p.chunks_per_row ? cls[4 * (uint64_t)c + k] : 0u;
+      incl[k] = wave_incl_scan(v[k], lane);
+      if (lane == 63) wsum[k][wave] = incl[k];
+    }
+    __syncthreads();
+    for (int k = 0; k < 3; ++k) {
+      unsigned long long before = incl[k] - v[k];
+      for (int w = 0; w < wave; ++w) before += wsum[k][w];
+      if (c < p.chunks_per_row) off[4 * (uint64_t)c + k] = carry[k] + before;
+      carry[k] += wsum[k][0] + wsum[k][1] + wsum[k][2] + wsum[k][3];
+    }
+  }
+}
+
+// The split pass of partition / argpartition.  grid: n_chunks, NT threads.  Every workgroup
+// walks its chunk in tiles of NT * IPT values; the values of a tile are brought into the
+// order below / equal / above in LDS (each class in input order: lane ranks from ballots,
+// wavefront offsets from a scan over the counts per load slot and wavefront) and written out
+// from there to the three places of the chunk, consecutive threads to consecutive addresses,
+// so that lines are written whole except where a class ends within the tile.  What travels is
+// the value as it came in (the key only decides the class), or, with POS, its position in the
+// row, staged as a 16-bit place within the tile.
+template <typename KeyT, bool POS, int NT, int IPT>
+__global__ void __launch_bounds__(NT)
+select_split_kernel(SelectParams<KeyT> p, KeyT* __restrict__ values_out, int64_t* __restrict__ pos_out,
+                    int64_t index_offset)
+{
+  constexpr int NW = NT / 64, T = NT * IPT;
+  static_assert(T <= 65536 && 2 * IPT * NW <= NT && (IPT * NW) % 64 == 0, "tile geometry");
+  using StageT = typename std::conditional<POS, uint16_t, KeyT>::type;
+  __shared__ __attribute__((aligned(16))) StageT stage[T];
+  __shared__ uint32_t cnt[2][IPT * NW];  // per class (below, equal): count per (load slot, wavefront)
+  __shared__ uint32_t tot[2];
+  const uint32_t row = blockIdx.x / p.chunks_per_row, chunk = blockIdx.x % p.chunks_per_row;
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const KeyT kth     = p.prefix[row];
+  uint64_t b0 = (uint64_t)chunk * p.chunk_len, b1 = b0 + p.chunk_len;
+  if (b1 > p.row_len) b1 = p.row_len;
+  if (b0 > b1) b0 = b1;
+  const KeyT* in = p.in + (uint64_t)row * p.row_len;
+  unsigned long long g[3];
+  for (int k = 0; k < 3; ++k) g[k] = p.chunk_off[4 * (uint64_t)blockIdx.x + k];
+  const uint64_t lane_lt = (1ull << lane) - 1;
+
+  for (uint64_t t0 = b0; t0 < b1; t0 += T) {
+    const uint32_t valid = b1 - t0 < (uint64_t)T ? (uint32_t)(b1 - t0) : (uint32_t)T;
+    KeyT raw[IPT];
+    uint32_t cls[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e = i * NT + tid;
+      raw[i]           = e < valid ? in[t0 + e] : KeyT{};
+    }
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e = i * NT + tid;
+      const KeyT k     = KeyOps<KeyT>::to_key(raw[i], p.xform);
+      cls[i]           = e >= valid ? 3u : key_lt(k, kth) ? 0u : key_eq(k, kth) ? 1u : 2u;
+      const uint64_t m0 = __ballot(cls[i] == 0), m1 = __ballot(cls[i] == 1);
+      if (lane == 0) {
+        cnt[0][i * NW + wave] = __popcll(m0);
+        cnt[1][i * NW + wave] = __popcll(m1);
+      }
+    }
+    __syncthreads();
+    // exclusive scan of the counts of each class in the order (load slot, wavefront): the
+    // first two wavefronts take a class each, IPT * NW / 64 counts per lane
+    if (wave < 2) {
+      constexpr int PER = IPT * NW / 64;
+      uint32_t v[PER], sum = 0;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        v[j] = cnt[wave][lane * PER + j];
+        sum += v[j];
+      }
+      const uint32_t incl = wave_incl_scan_u32(sum);
+      uint32_t run        = incl - sum;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        cnt[wave][lane * PER + j] = run;
+        run += v[j];
+      }
+      if (lane == 63) tot[wave] = incl;
+    }
+    __syncthreads();
+    const uint32_t n0 = tot[0], n1 = tot[1];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e  = i * NT + tid;
+      const uint64_t m0 = __ballot(cls[i] == 0), m1 = __ballot(cls[i] == 1);
+      const uint32_t before0 = cnt[0][i * NW + wave] + __popcll(m0 & lane_lt);
+      const uint32_t before1 = cnt[1][i * NW + wave] + __popcll(m1 & lane_lt);
+      const uint32_t at = cls[i] == 0 ? before0 : cls[i] == 1 ? n0 + before1 : n0 + n1 + (e - before0 - before1);
+      if (cls[i] < 3) {
+        if constexpr (POS) stage[at] = (uint16_t)e;
+        else stage[at] = raw[i];
+      }
+    }
+    __syncthreads();
+    const int64_t tile_pos = (int64_t)t0 + index_offset;
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e = i * NT + tid;
+      if (e < valid) {
+        const unsigned long long dst = e < n0 ? g[0] + e : e < n0 + n1 ? g[1] + (e - n0) : g[2] + (e - n0 - n1);
+        if constexpr (POS) pos_out[dst] = tile_pos + (int64_t)stage[e];
+        else values_out[dst] = stage[e];
+      }
+    }
+    g[0] += n0;
+    g[1] += n1;
+    g[2] += valid - n0 - n1;
+  }
 }
 
 // grid: n_chunks, after the last pick; keys of at most 8 bytes.  For callers that want the

@@ -62,6 +62,29 @@ def test_partition_and_argpartition_long_rows(dtype):
         assert_partitioned(a, b, n // 2)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128],
+                         ids=lambda d: np.dtype(d).name)
+def test_values_keep_their_bit_patterns(dtype):
+    """The split moves the values as they came in: NaN payloads and signed zeros survive."""
+    rng = np.random.default_rng(55)
+    n = 120001
+    a = random_array(dtype, n, rng)
+    size = a.dtype.itemsize
+
+    def bit_patterns(x):
+        raw = np.ascontiguousarray(x).tobytes()
+        return sorted(raw[i:i + size] for i in range(0, len(raw), size))
+
+    want = bit_patterns(a)
+    for kth in (0, n // 2, n - 1):
+        out = np.asarray(num.partition(a, kth))
+        assert_partitioned(a, out, kth)
+        assert bit_patterns(out) == want
+    b = num.array(a)
+    b.partition(n // 3)
+    assert bit_patterns(np.asarray(b)) == want
+
+
 def test_rows_axes_and_fallbacks():
     rng = np.random.default_rng(52)
     a = rng.standard_normal((3, 70001)).astype(np.float32)
