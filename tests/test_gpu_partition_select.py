@@ -85,6 +85,19 @@ def test_values_keep_their_bit_patterns(dtype):
     assert bit_patterns(np.asarray(b)) == want
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.int64], ids=lambda d: np.dtype(d).name)
+def test_many_rows(dtype):
+    """Hundreds of rows just long enough for the selection: few chunks per row."""
+    rng = np.random.default_rng(56)
+    rows, n = 300, 66001
+    a = random_array(dtype, rows * n, rng).reshape(rows, n)
+    for kth in (0, n // 2, n - 1):
+        assert_partitioned(a, num.partition(a, kth, axis=1), kth)
+        idx = np.asarray(num.argpartition(a, kth, axis=1))
+        assert np.array_equal(np.sort(idx, axis=1), np.broadcast_to(np.arange(n), a.shape))
+        assert_partitioned(a, np.take_along_axis(a, idx, axis=1), kth)
+
+
 def test_rows_axes_and_fallbacks():
     rng = np.random.default_rng(52)
     a = rng.standard_normal((3, 70001)).astype(np.float32)

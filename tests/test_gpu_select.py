@@ -86,6 +86,18 @@ def test_rows_that_narrow_down_at_different_passes(abi, dtype):
         assert same_values(k, s[:, kth]) and same_values(nxt, s[:, kth + 1]) and same_values(top, s[:, -1])
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.int64], ids=lambda d: np.dtype(d).name)
+def test_many_rows(abi, dtype):
+    """Hundreds of rows just long enough for the selection: few chunks per row."""
+    rng = np.random.default_rng(64)
+    rows, n = 300, 66001
+    a = random_array(dtype, rows * n, rng).reshape(rows, n)
+    s = np.sort(a, axis=1)
+    for kth in (0, n // 2, n - 2):
+        k, nxt, top = select(abi, a, kth)
+        assert same_values(k, s[:, kth]) and same_values(nxt, s[:, kth + 1]) and same_values(top, s[:, -1])
+
+
 def test_nan_rows_and_signed_zeros(abi):
     rng = np.random.default_rng(63)
     n = 70001
