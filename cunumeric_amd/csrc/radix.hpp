@@ -906,8 +906,50 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
       // value that the wave has seen before this lane (earlier wave-rows, lower lanes of this
       // one), because the LDS of this GPU serves the lanes of one instruction that hit the
       // same word in lane order (see rank_by_add above).
+      // A wave-row whose 64 keys hold one or two digit values (runs of equal keys, which the
+      // earlier passes have brought together) would queue up on one or two counters, 64 deep
+      // in all: there the first lane of each group adds the group's size and the rank is the
+      // value it gets plus the number of lower lanes of the group.  Looking for such rows
+      // costs more than the add itself, so the first and the last wave-row of the tile are
+      // asked first, and the others only if one of the two is such a row.
+      struct Groups {
+        bool grouped;     // the row holds at most two digit values (same in every lane)
+        bool first;       // this lane belongs to the group of lane 0
+        uint32_t second;  // first lane of the other group (0 if there is none)
+        uint64_t mine;    // the lanes of this lane's group
+      };
+      auto groups_of = [&](uint32_t d) {
+        Groups g;
+        const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+        const uint64_t m0 = __ballot(d == d0);
+        g.second          = ~m0 ? (uint32_t)__builtin_ctzll(~m0) : 0u;
+        const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d, (int)g.second);
+        const uint64_t m1 = __ballot(d == d1);
+        g.grouped         = (m0 | m1) == ~0ull;
+        g.first           = d == d0;
+        g.mine            = g.first ? m0 : m1;
+        return g;
+      };
+      if (groups_of(digit_of(ck[0])).grouped || groups_of(digit_of(ck[IPT - 1])).grouped) {
 #pragma unroll
-      for (int i = 0; i < IPT; ++i) rank[i] = atomicAdd(&my_hist[digit_of(ck[i])], 1u);
+        for (int i = 0; i < IPT; ++i) {
+          const uint32_t d = digit_of(ck[i]);
+          const Groups g   = groups_of(d);
+          uint32_t r       = 0;
+          if (!g.grouped || lane == (g.first ? 0u : g.second))
+            r = atomicAdd(&my_hist[d], g.grouped ? (uint32_t)__popcll(g.mine) : 1u);
+          if (g.grouped) {
+            const uint32_t r0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
+            const uint32_t r1 = (uint32_t)__builtin_amdgcn_readlane((int)r, (int)g.second);
+            r = (g.first ? r0 : r1) +
+                __builtin_amdgcn_mbcnt_hi((uint32_t)(g.mine >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)g.mine, 0u));
+          }
+          rank[i] = r;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < IPT; ++i) rank[i] = atomicAdd(&my_hist[digit_of(ck[i])], 1u);
+      }
     } else {
     auto finish_rank = [&](int i, uint32_t d, uint32_t plo, uint32_t phi) {
       const uint32_t below = __builtin_amdgcn_mbcnt_hi(phi, __builtin_amdgcn_mbcnt_lo(plo, 0u));

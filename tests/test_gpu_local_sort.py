@@ -51,6 +51,30 @@ def test_heavy_ties(abi, dtype):
     assert np.array_equal(got, np.argsort(a, kind="stable"))
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64], ids=lambda d: np.dtype(d).name)
+@pytest.mark.parametrize("copies", [16, 40, 64, 100, 256, 1000])
+def test_runs_of_equal_keys_with_spread_out_digits(abi, dtype, copies):
+    """Values drawn from a pool of distinct random values: every digit value is about equally
+    frequent, so the scatter ranks by returning LDS adds, and the later passes meet runs of
+    `copies` equal keys, where wave-rows of one or two digit values are ranked group-wise."""
+    rng = np.random.default_rng(14)
+    n = 1 << 20
+    if np.dtype(dtype).kind == "f":
+        pool = rng.standard_normal(n // copies).astype(dtype) * 1e3
+    else:
+        ii = np.iinfo(dtype)
+        pool = rng.integers(ii.min, ii.max, n // copies, dtype=dtype)
+    a = pool[rng.integers(0, pool.size, n)]
+    print(f"runs dtype={np.dtype(dtype).name} copies={copies}", flush=True)
+    got = abi.local_sort(a, n, argsort=True)
+    assert np.array_equal(got, np.argsort(a, kind="stable"))
+    assert bits_equal(abi.local_sort(a, n, argsort=False), np.sort(a, kind="stable"))
+    # two rows, so that a row starts in the middle of a tile
+    b = a[: 2 * 300007].reshape(2, 300007)
+    got = abi.local_sort(b, 300007, argsort=True).reshape(2, -1)
+    assert np.array_equal(got, np.argsort(b, axis=1, kind="stable"))
+
+
 @pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float16, np.float32, np.int64, np.float64,
                                    np.complex128], ids=lambda d: np.dtype(d).name)
 @pytest.mark.parametrize("rows,row_len", [(7, 5000), (3, 12288), (64, 4096), (5, 1), (1000, 17),
