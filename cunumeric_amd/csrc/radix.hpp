@@ -554,13 +554,27 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
     next_shift = plan.next_shift;
     if (p.key_bits) {
       const bool cur = input_buffer(p, plan) != 0;
+      // (The chosen pointers are the same in every lane.  In the kernels with 16 keys per
+      // thread, which have no vector register to spare, saying so keeps them in scalar
+      // registers; left to the compiler they pushed other values out to scratch memory there.
+      // The other kernels were measured slower with it and keep the plain form.)
+      auto chosen = [](auto* q) {
+        if constexpr (IPT >= 16) {
+          const unsigned long long v = (unsigned long long)q;
+          const uint32_t a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+          const uint32_t b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+          return (decltype(q))(((unsigned long long)b << 32) | a);
+        } else {
+          return q;
+        }
+      };
       if (!FIRST) {
-        p.keys_in = cur ? p.key_buf[1] : p.key_buf[0];
-        p.pay_in  = cur ? p.pay_buf[1] : p.pay_buf[0];
+        p.keys_in = chosen(cur ? p.key_buf[1] : p.key_buf[0]);
+        p.pay_in  = chosen(cur ? p.pay_buf[1] : p.pay_buf[0]);
       }
       if (!LAST) {
-        p.keys_out = cur ? p.key_buf[0] : p.key_buf[1];
-        p.pay_out  = cur ? p.pay_buf[0] : p.pay_buf[1];
+        p.keys_out = chosen(cur ? p.key_buf[0] : p.key_buf[1]);
+        p.pay_out  = chosen(cur ? p.pay_buf[0] : p.pay_buf[1]);
       }
     }
   }

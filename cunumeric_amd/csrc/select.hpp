@@ -28,7 +28,6 @@
 namespace misort {
 
 constexpr int SEL_NT = 512;
-constexpr int SEL_U  = 8;  // 16-byte loads a lane keeps in flight in the histogram pass
 // where the histogram pass of a row reads its keys, and whether it writes candidates
 constexpr uint32_t SEL_ROW = 0, SEL_APPEND = 1, SEL_CAND = 2;
 
@@ -124,6 +123,9 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
   struct alignas(16) Vec {
     KeyT v[V];
   };
+  // 16-byte loads a lane keeps in flight (fewer for 1-byte keys, whose 16 counts per load
+  // would not fit the registers otherwise)
+  constexpr int U = sizeof(KeyT) == 1 ? 2 : 8;
   // (one instance of the loop per state, so that the plain pass carries none of the rest)
   auto scan = [&](auto state_tag) {
     constexpr uint32_t ST = decltype(state_tag)::value;
@@ -164,10 +166,10 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
     uint64_t i0 = b0;
     if (V > 1 && (reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
       uint64_t nvec = (b1 - b0) / V;
-      if (ST == SEL_APPEND) nvec -= nvec % ((uint64_t)SEL_NT * SEL_U);
+      if (ST == SEL_APPEND) nvec -= nvec % ((uint64_t)SEL_NT * U);
       const Vec* vb = reinterpret_cast<const Vec*>(base + b0);
       if constexpr (sizeof(Vec) == 16) {
-        stream_vectors<SEL_U>(vb, nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
+        stream_vectors<U>(vb, nvec, threadIdx.x, SEL_NT, [&](const Vec& r) {
 #pragma unroll
           for (int e = 0; e < V; ++e) count(r.v[e], true);
           flush_if_full();
