@@ -136,23 +136,36 @@ def _select_rows(a: ndarray, k: int, want_next: bool):
 
 def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool):
     """``a`` has the reduction axis last: the samples at the sorted positions ``wanted`` of
-    every row, as tensors of the row shape, and (or None) which rows hold a NaN.  One or two
-    adjacent positions on long rows are found by selection: two or three reads of the rows
-    instead of a sort, and the rows' largest element, which comes with it, tells the NaNs.
-    Anything else sorts the rows."""
+    every row, as tensors of the row shape, and (or None) which rows hold a NaN.  A few
+    positions on long rows are found by selection, one call per position or adjacent pair: two
+    reads of the rows each instead of a sort (which moves them once or twice per key byte), and
+    the rows' largest element, which comes with it, tells the NaNs.  Anything else sorts the
+    rows."""
     from .module import sort
 
     n = a.shape[-1]
     wanted = sorted(set(wanted))
-    if (len(wanted) <= 2 and wanted[-1] - wanted[0] <= 1 and n >= (1 << 16) and a.dtype.itemsize >= 4 and
+    pairs: list[tuple[int, bool]] = []  # (position, the next one is wanted too)
+    for k in wanted:
+        if pairs and pairs[-1][0] + 1 == k and not pairs[-1][1]:
+            pairs[-1] = (k - 1, True)
+        elif not (pairs and pairs[-1][1] and pairs[-1][0] + 1 == k):
+            pairs.append((k, False))
+    # a selection costs about two reads of the rows, a sort two (one read, one write) per key byte
+    if (0 < len(pairs) <= a.dtype.itemsize // 2 + 1 and n >= (1 << 16) and a.dtype.itemsize >= 4 and
             a.dtype.kind in "fiu" and a.size):
-        k = wanted[0]
-        found = _select_rows(a, k, len(wanted) == 2)
-        if found is not None:
-            out = {k: found[0]}
-            if len(wanted) == 2:
+        out: dict[int, torch.Tensor] = {}
+        top = None
+        for k, with_next in pairs:
+            found = _select_rows(a, k, with_next)
+            if found is None:
+                break
+            out[k] = found[0]
+            if with_next:
                 out[k + 1] = found[1]
-            return out, (torch.isnan(found[-1]) if a.dtype.kind == "f" else None)
+            top = found[-1]
+        else:
+            return out, (torch.isnan(top) if a.dtype.kind == "f" else None)
     if overwrite_input:
         a.sort(axis=-1)
         s = a
