@@ -8,9 +8,9 @@ count the non-NaN elements of every slice, sort with the NaNs moved behind every
 :8647-8754).
 
 Same arguments, result shapes / dtypes and exceptions.  The order statistics come from the
-GPU sort of this package; for ONE quantile over a flat array or long rows they come from the
-selection behind ``partition`` instead (the reference's own comment at :8462-8467 names that
-as the cheaper way it does not take).  Picking the two neighbours out of the sorted array
+GPU sort of this package; for a few quantiles over a flat array or long rows they come from the
+selection behind ``partition`` instead, which moves no row (the reference's own comment at
+:8462-8467 names partitioning as the cheaper way it does not take).  Picking the two neighbours out of the sorted array
 and blending them is elementwise arithmetic, which is not part of the sort path: it runs
 through torch on the device.  NumPy defines the 13 methods (numpy.quantile); the position of
 a quantile in the sorted sample and its blending weight follow NumPy's definitions, so
