@@ -343,10 +343,12 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.tiles_per_row = (pl.row_len + pl.tile - 1) / pl.tile;
     size_t target = target_chunks;
     if (target == 0) {
-      // two workgroups per CU; one when that still leaves a workgroup fewer than four tiles
-      // (measured: 2^24 int32 values 4 % faster, 2^26 and up 5 % slower with one)
+      // two workgroups per CU, which balances the end of a long pass (2^28 keys: 1-3 % faster
+      // than one); one per CU below 32 tiles per workgroup at two, where paying a workgroup's
+      // start-up once per CU counts for more (2^24 (key, position) pairs 7 % faster with one,
+      // 2^25 4 %, 2^26 3 %; level at 32 tiles)
       target = kTargetChunks;
-      if (pl.rows * pl.tiles_per_row < 4 * target) target /= 2;
+      if (pl.rows * pl.tiles_per_row < 32 * target) target /= 2;
     }
     size_t want = (target + pl.rows - 1) / pl.rows;  // chunks per row aimed at
     if (want < 1) want = 1;
