@@ -556,8 +556,9 @@ __global__ void __launch_bounds__(SEL_NT) select_above_kernel(SelectParams<KeyT>
     i0 = b0 + nvec * V;
   }
   for (uint64_t i = i0 + threadIdx.x; i < b1; i += SEL_NT) look(base[i]);
-  // (a key above the kth key that is all ones leaves the word as it is: all ones)
-  unsigned long long lo = above;
+  // (Nothing found, or only a key that is all ones: the word stays all ones in its full 64
+  // bits, whatever the width of the key, which is what the second launch asks for.)
+  unsigned long long lo = above == (KeyT)~(KeyT)0 ? ~0ull : (unsigned long long)above;
 #pragma unroll
   for (int s = 32; s > 0; s >>= 1) {
     const unsigned long long l2 = __shfl_xor(lo, s, 64);

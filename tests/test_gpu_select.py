@@ -8,6 +8,7 @@ and a NaN as the default NaN, which is what the entry point documents)."""
 import numpy as np
 import pytest
 
+from oracle import misort_oracle as oracle
 from tests.util import Abi, random_array
 
 pytestmark = pytest.mark.gpu
@@ -96,6 +97,29 @@ def test_many_rows(abi, dtype):
     for kth in (0, n // 2, n - 2):
         k, nxt, top = select(abi, a, kth)
         assert same_values(k, s[:, kth]) and same_values(nxt, s[:, kth + 1]) and same_values(top, s[:, -1])
+
+
+@pytest.mark.parametrize("dtype", [np.uint32, np.int32, np.float32, np.int64, np.float64],
+                         ids=lambda d: np.dtype(d).name)
+def test_next_element_lies_outside_the_keys_that_still_match(abi, dtype):
+    """Keys spread so thinly that the kth key is the largest of those sharing its leading
+    byte: the element after it is not among the keys the selection kept, and is found by
+    reading the row once more."""
+    rng = np.random.default_rng(65)
+    n = 70001
+    step = 60000 if np.dtype(dtype).itemsize == 4 else 1 << 46
+    vals = (np.arange(n, dtype=np.int64) - (n // 2 if np.dtype(dtype).kind != "u" else 0)) * step
+    if dtype == np.int32:
+        vals //= 2
+    a = np.stack([rng.permutation(vals).astype(dtype) for _ in range(3)])
+    s = np.sort(a, axis=1)
+    key = oracle.to_key(s[0])[-1]  # the sort keys of row 0, ascending
+    shift = key.dtype.itemsize * 8 - 8
+    last_of_bucket = np.nonzero((key[:-1] >> shift) != (key[1:] >> shift))[0]
+    assert last_of_bucket.size >= 4
+    for kth in [int(k) for k in last_of_bucket[:: max(1, last_of_bucket.size // 6)]] + [n - 2]:
+        k, nxt, top = select(abi, a, kth)
+        assert same_values(k, s[:, kth]) and same_values(nxt, s[:, kth + 1]) and same_values(top, s[:, -1]), kth
 
 
 def test_nan_rows_and_signed_zeros(abi):
