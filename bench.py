@@ -178,7 +178,7 @@ WORKLOADS = {
     "c4": ("C4: 1-D int64, 16 distinct values (Zipf 1.2), stable argsort", make_c4, 28, True, 0),
     "c5a": ("C5a: 1-D complex64, 1024 distinct real parts, stable argsort", make_c5a, 26, True, 0),
     "c5b": ("C5b: 1-D float16 uniform(-1,1), sort (keys only)", make_c5b, 30, False, 0),
-    "i64small": ("1-D int64 below 50000, stable argsort (five of the eight radix passes see one "
+    "i64small": ("1-D int64 below 50000, stable argsort (six of the eight radix passes see one "
                  "digit value and are skipped)", make_small_int64, 28, True, 0),
 }
 
@@ -741,15 +741,29 @@ def main() -> int:
         # the time an event takes between launches, so the sum over the kernels is an upper
         # bound of the call (call_ms, timed without the inner events, is the figure to use).
         # A radix pass over a digit that no key varies in is skipped on the device: its two
-        # launches return at once.  They are counted apart (launches whose median duration is
-        # below a twentieth of the longest launch of the same kernel), so that the averages and
+        # launches return at once, and so does, in large sorts, the last-pass form of the
+        # scatter that is launched beside every middle pass in case the digits after it are
+        # constant.  They are counted apart (launches whose median duration is
+        # below a twentieth of the longest upsweep / scatter launch), so that the averages and
         # the roofline below are those of the passes that ran (P executed, not P planned).
         kernels = {}
+        medians = {name: np.median(np.asarray(v, dtype=np.float64).reshape(reps, -1), axis=0)
+                   for name, v in acc.items()}
+        longest_scatter = max([m.max() for name, m in medians.items() if name.startswith("downsweep_")] or [0.0])
         for name, v in acc.items():
             per_call = np.asarray(v, dtype=np.float64).reshape(reps, -1)
-            per_launch = np.median(per_call, axis=0)
-            ran = per_launch >= 0.05 * per_launch.max() if name in ("upsweep", "downsweep_middle") else \
-                np.ones_like(per_launch, dtype=bool)
+            per_launch = medians[name]
+            if name == "upsweep":
+                ran = per_launch >= 0.05 * per_launch.max()
+            elif name in ("downsweep_middle", "downsweep_last"):
+                ran = per_launch >= 0.05 * longest_scatter
+            else:
+                ran = np.ones_like(per_launch, dtype=bool)
+            if not ran.any():  # (every launch of this role returned at once)
+                kernels[name] = {"launches_per_step": 0, "avg_ms": 0.0,
+                                 "skipped_launches_per_step": int(per_launch.size),
+                                 "skipped_avg_ms": float(per_launch.mean())}
+                continue
             kernels[name] = {"launches_per_step": int(ran.sum()),
                              "avg_ms": float(np.median(per_call[:, ran].mean(axis=1)))}
             if not ran.all():
@@ -776,6 +790,8 @@ def main() -> int:
             else:
                 continue
             l = kk["launches_per_step"]
+            if l == 0:
+                continue
             tot_bytes += b * n * l
             tot_ms += kk["avg_ms"] * l
             n_launch += l

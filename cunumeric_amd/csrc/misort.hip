@@ -62,6 +62,16 @@ static bool skip_passes_default()
   return v;
 }
 
+// From how many bytes of keys on the last pass whose digit varies writes the result (it costs
+// one more launch per middle pass).  MISORT_EARLY_LAST_BYTES in the environment overrides the
+// 256 MB; read at every call, so that tests can reach the path with small arrays.
+static size_t early_last_min_bytes()
+{
+  const char* e = getenv("MISORT_EARLY_LAST_BYTES");
+  if (e && *e) return (size_t)strtoull(e, nullptr, 10);
+  return (size_t)1 << 28;
+}
+
 static int fail(int code, const std::string& msg)
 {
   g_last_error = msg;
@@ -251,6 +261,7 @@ struct Plan {
   // middle passes whose digit is the same in every key are skipped (decided on the device from
   // the OR of the keys and of their complements, which the first upsweep leaves in key_bits)
   bool skip_dead_passes = false;
+  bool early_last = false;  // the last pass whose digit varies writes the result (large sorts only)
   size_t off_key_bits = 0;
   size_t off_gather_idx = 0, off_gather_src = 0;
   // counting sort of 2-byte keys: chunks of the histogram kernel, counters, their scan
@@ -390,6 +401,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // (not for keys-only float sorts: the patch of their zeros and NaNs counts on which of the
     // two buffers the last pass leaves free)
     pl.skip_dead_passes = skip_passes_default() && pl.n_passes >= 3 && !pl.specials;
+    // (one more launch per middle pass, about 5 us each: from 256 MB of keys on)
+    pl.early_last = pl.skip_dead_passes && pl.volume * pl.dt.bytes >= early_last_min_bytes();
     pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
     pl.side_adaptive = side_band_default() && !pl.side_band && pl.n_passes >= 2 && pl.dt.bytes >= 4 &&
                        (pl.pay != PAY_NONE || pl.dt.bytes > 4);
@@ -572,6 +585,24 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   pp.pay_buf[0]      = PAY != PAY_NONE ? S + pl.off_pay[0] : nullptr;
   pp.pay_buf[1]      = PAY != PAY_NONE ? S + pl.off_pay[1] : nullptr;
 
+  // where the pass that writes the result puts it
+  void* final_keys = nullptr;
+  void* final_pay  = nullptr;
+  if (pl.gather_values)
+    final_keys = nullptr;
+  else if (alias_keys)
+    final_keys = S + pl.off_keys[0];
+  else
+    final_keys = write_keys_last ? vout : nullptr;
+  if (PAY != PAY_NONE) {
+    if (pl.gather_values)
+      final_pay = S + pl.off_gather_idx;
+    else if (alias_pay)
+      final_pay = S + pl.off_pay[0];
+    else
+      final_pay = iout;
+  }
+
   const void* cur_keys = vin;
   const void* cur_pay  = iin;
   for (int pass = 0; pass < pl.n_passes; ++pass) {
@@ -579,20 +610,8 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
     void* dst_keys;
     void* dst_pay = nullptr;
     if (last) {
-      if (pl.gather_values)
-        dst_keys = nullptr;
-      else if (alias_keys)
-        dst_keys = S + pl.off_keys[0];
-      else
-        dst_keys = write_keys_last ? vout : nullptr;
-      if (PAY != PAY_NONE) {
-        if (pl.gather_values)
-          dst_pay = S + pl.off_gather_idx;
-        else if (alias_pay)
-          dst_pay = S + pl.off_pay[0];
-        else
-          dst_pay = iout;
-      }
+      dst_keys = final_keys;
+      dst_pay  = final_pay;
     } else {
       dst_keys = S + pl.off_keys[pass & 1];
       if (PAY != PAY_NONE) dst_pay = S + pl.off_pay[pass & 1];
@@ -615,12 +634,24 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
       unsigned long long* bits = reinterpret_cast<unsigned long long*>(S + pl.off_key_bits);
       pp.key_bits_out = (pl.skip_dead_passes && first) ? bits : nullptr;
       pp.key_bits     = pl.skip_dead_passes ? bits : nullptr;  // complete once the first upsweep has run
+      pp.early_last   = pl.early_last ? 1 : 0;
     }
     pp.slab_tot = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + (pass & 1) * pl.slab_tot_bytes);
     pp.slab_tot_next =
       last ? nullptr
            : reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + ((pass + 1) & 1) * pl.slab_tot_bytes);
     launch_pass<KeyT, PAY>(L, pl, first, last, pp);
+    if (pl.early_last && !first && !last) {
+      // If no key varies in any digit after this one, this pass writes the result: the same
+      // scatter in its last-pass form, which returns at once otherwise (as the form above
+      // does in that case).
+      PassParams pe    = pp;
+      pe.keys_out      = final_keys;
+      pe.pay_out       = final_pay;
+      pe.digits_out    = nullptr;
+      pe.slab_tot_next = nullptr;
+      launch_downsweep<KeyT, PAY>(L, pl, K_DOWN_LAST, false, true, pe);
+    }
 
     if constexpr (is_float_width<KeyT>() && PAY == PAY_NONE) {
       if (pl.specials && first) {
@@ -1192,7 +1223,8 @@ int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int arg
            (int)pl.gather_values, pl.side_band ? 1 : (pl.side_adaptive ? 2 : 0), pl.total);
   if (pl.skip_dead_passes) {
     const size_t len = strlen(buf);
-    if (len + 16 < buf_bytes) snprintf(buf + len, buf_bytes - len, " skip_dead_passes=1");
+    if (len + 32 < buf_bytes)
+      snprintf(buf + len, buf_bytes - len, " skip_dead_passes=1%s", pl.early_last ? " early_last=1" : "");
   }
   return MISORT_OK;
 }

@@ -10,8 +10,8 @@
 //                     the digit values and over the chunks before its own (where its keys of
 //                     each digit value start), then it walks its tiles in order, carrying the
 //                     running start of every digit value, so no workgroup ever waits on another.
-// Middle passes whose digit is the same in every key are skipped: the first upsweep ORs the
-// keys and their complements, every later kernel works out the rest from those words
+// Passes after the first whose digit is the same in every key are skipped: the first upsweep
+// ORs the keys and their complements, every later kernel works out the rest from those words
 // (plan_pass).
 // Keys-only sorts of 8-byte elements: every pass but the last also writes the next pass's digit
 // of each key as a byte (SIDE), which the next upsweep counts instead of the keys
@@ -77,6 +77,7 @@ struct PassParams {
   unsigned long long* key_bits_out;
   void* key_buf[2];
   void* pay_buf[2];
+  int early_last;  // leading digits that no key varies in are left out too: see plan_pass
   const void* pay_in;    // PAY_IDX32: u32 (ignored when FIRST); PAY_I64: int64, NULL => positions
   void* pay_out;         // PAY_IDX32: u32, int64 when LAST; PAY_I64: int64
   uint32_t* chunk_hist;             // [rows * chunks_per_row][RADIX] counts of this pass
@@ -104,14 +105,21 @@ constexpr int KEY_BITS_SLOTS = 8;
 // What a kernel of pass p.pass works out from key_bits (all of it uniform).
 struct PassPlan {
   bool skip;        // this pass moves nothing
+  bool is_last;     // this is the last pass that moves anything: it writes the result
   uint32_t parity;  // dead passes before this one, modulo 2: the ping-pong buffers are swapped
   int next_shift;   // digit position of the next live pass
   int prev_live;    // the last live pass before this one
   int const_digit;  // the digit value every key has in this pass, or -1 if the digit varies
 };
+// Pass 0 transforms the elements into keys and is never skipped.  The pass over the most
+// significant digit transforms them back: without early_last it always runs (and skips the
+// counting if its digit is constant); with early_last the last pass whose digit varies
+// writes the result instead (the host launches, for every pass after the first, the scatter
+// kernel in both forms, and each finds out here whether it is the one to run), unless that
+// would be pass 0, which cannot be first and last at once when it sorts in place.
 __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
 {
-  PassPlan r{false, 0u, p.shift + RADIX_BITS, p.pass - 1, -1};
+  PassPlan r{false, p.pass == p.n_passes - 1, 0u, p.shift + RADIX_BITS, p.pass - 1, -1};
   if (!p.key_bits) return r;
   auto uniform64 = [](unsigned long long v) {  // same in every lane: keep it in scalar registers
     const uint32_t a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
@@ -126,23 +134,30 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
   }
   const unsigned long long lo = uniform64(w[0] & w[2]);
   const unsigned long long hi = uniform64(w[1] & w[3]);
-  auto dead = [&](int j) {  // first and last pass transform the elements: never skipped
-    if (j <= 0 || j >= p.n_passes - 1) return false;
+  auto constant = [&](int j) {  // no key varies in digit j
     const unsigned long long w = j < 8 ? lo : hi;
     return ((w >> (8 * (j & 7))) & 0xFFull) == 0;
   };
+  // the last pass that runs
+  int last = p.n_passes - 1;
+  if (p.early_last) {
+    while (last > 0 && constant(last)) --last;
+    if (last == 0) last = p.n_passes - 1;
+  }
+  auto dead = [&](int j) { return j > last || (j > 0 && j < last && constant(j)); };
   for (int j = 1; j < p.pass; ++j) r.parity ^= dead(j) ? 1u : 0u;
-  r.skip = dead(p.pass);
+  r.skip    = dead(p.pass);
+  r.is_last = p.pass == last;
   int nx = p.pass + 1;
-  while (dead(nx)) ++nx;
+  while (nx < last && dead(nx)) ++nx;
   r.next_shift = nx * RADIX_BITS;
   int pv = p.pass - 1;
-  while (dead(pv)) --pv;
+  while (pv > 0 && dead(pv)) --pv;
   r.prev_live = pv;
   {
-    const unsigned long long vary = p.pass < 8 ? lo : hi, ones = uniform64(p.pass < 8 ? w[0] : w[1]);
+    const unsigned long long ones = uniform64(p.pass < 8 ? w[0] : w[1]);
     const int sh = 8 * (p.pass & 7);
-    if (((vary >> sh) & 0xFFull) == 0) r.const_digit = (int)((ones >> sh) & 0xFFull);
+    if (constant(p.pass)) r.const_digit = (int)((ones >> sh) & 0xFFull);
   }
   return r;
 }
@@ -551,6 +566,8 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
         p.slab_tot_next[((uint64_t)row * p.slabs_per_row + chunk) * RADIX + tid] = 0;
       return;
     }
+    // the pass that writes the result is launched in both forms: only the LAST one runs
+    if (plan.is_last != LAST) return;
     next_shift = plan.next_shift;
     if (p.key_bits) {
       const bool cur = input_buffer(p, plan) != 0;

@@ -80,7 +80,9 @@ const char* misort_last_error(void);
  * count reads bytes instead of keys); MISORT_SIDE_BAND=0 in the environment before the first
  * call into the library leaves it out (give the query and the sort the same environment).
  * Radix passes over a digit that is the same in every key are skipped (decided on the device,
- * nothing is read back); MISORT_SKIP_PASSES=0 runs them all.
+ * nothing is read back); MISORT_SKIP_PASSES=0 runs them all.  Sorts of 256 MB of keys and
+ * more also leave out the passes over constant most significant digits (the last pass whose
+ * digit varies writes the result); MISORT_EARLY_LAST_BYTES=<bytes> moves that limit.
  */
 size_t misort_scratch_bytes(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                             int has_indices_in);

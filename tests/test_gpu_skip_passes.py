@@ -1,6 +1,9 @@
 """Radix passes over a digit that is the same in every key are skipped on the device (the
 first upsweep ORs the keys and their complements; every later kernel derives from those
-words which middle passes are dead and which ping-pong buffer holds its input).  Inputs whose
+words which passes are dead and which ping-pong buffer holds its input).  Large sorts also
+leave out the passes over the most significant digits if those are constant: the last pass
+whose digit varies then writes the result; MISORT_EARLY_LAST_BYTES=0 makes small sorts do
+the same, which is how the tests below reach that path.  Inputs whose
 constant bytes sit in every combination of positions, for all key widths with middle passes,
 sorts and argsorts, rows, a caller payload, and the same input with the skipping switched
 off must agree with NumPy."""
@@ -21,6 +24,15 @@ def abi():
     return Abi()
 
 
+@pytest.fixture(params=[False, True], ids=["top pass kept", "last live pass writes the result"])
+def early_last(request, monkeypatch):
+    if request.param:
+        monkeypatch.setenv("MISORT_EARLY_LAST_BYTES", "0")
+    else:
+        monkeypatch.delenv("MISORT_EARLY_LAST_BYTES", raising=False)
+    return request.param
+
+
 def masked_random(dtype, n, rng, live_bytes):
     """Unsigned random values in which only the bytes listed in live_bytes vary; the others
     carry a fixed non-zero pattern."""
@@ -39,9 +51,10 @@ WIDTH8 = [(0,), (0, 1), (0, 7), (3, 4), (7,), (1, 2, 3, 4, 5, 6), (0, 2, 4, 6), 
 
 @pytest.mark.parametrize("dtype,patterns", [(np.uint32, WIDTH4), (np.int32, WIDTH4), (np.uint64, WIDTH8),
                                              (np.int64, WIDTH8)], ids=["uint32", "int32", "uint64", "int64"])
-def test_constant_bytes_in_every_position(abi, dtype, patterns):
+def test_constant_bytes_in_every_position(abi, dtype, patterns, early_last):
     rng = np.random.default_rng(61)
     n = 300007
+    assert ("early_last=1" in abi.describe_plan(dtype, n, n, True)) == early_last
     for live in patterns:
         a = masked_random(dtype, n, rng, live)
         for chunks in (0, 3):
@@ -52,7 +65,7 @@ def test_constant_bytes_in_every_position(abi, dtype, patterns):
 
 @pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float32, np.float64, np.complex64, np.complex128],
                          ids=lambda d: np.dtype(d).name)
-def test_small_ranges_rows_and_payload(abi, dtype):
+def test_small_ranges_rows_and_payload(abi, dtype, early_last):
     """Values from a small range (the usual case for integer data): the upper digits of the
     keys are constant.  Floats and complex numbers built from small integers have constant
     low mantissa bytes instead."""
@@ -76,7 +89,7 @@ def test_small_ranges_rows_and_payload(abi, dtype):
     assert bits_equal(got, np.sort(flat[:row_len], kind="stable"))
 
 
-def test_large_int64_small_range(abi):
+def test_large_int64_small_range(abi, early_last):
     rng = np.random.default_rng(63)
     n = 1 << 24
     a = rng.integers(0, 50000, n, dtype=np.int64)

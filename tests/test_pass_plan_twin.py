@@ -1,4 +1,4 @@
-"""CPU twin of plan_pass / input_buffer (cunumeric_amd/csrc/radix.hpp): which middle radix
+"""CPU twin of plan_pass / input_buffer (cunumeric_amd/csrc/radix.hpp): which radix
 passes are skipped and which of the two ping-pong buffers a pass reads, worked out by every
 kernel on its own from the bits that vary over the keys.  The twin restates the rule; the
 test walks a sort pass by pass for every set of dead passes and checks what the kernels rely
@@ -10,49 +10,65 @@ import itertools
 import pytest
 
 
-def plan(varying_bytes, pass_no, n_passes):
-    """(skip, parity, next_live, prev_live) as plan_pass computes them."""
+def plan(varying_bytes, pass_no, n_passes, early_last=False):
+    """(skip, parity, next_live, prev_live, is_last) as plan_pass computes them."""
+    last = n_passes - 1
+    if early_last:
+        while last > 0 and last not in varying_bytes:
+            last -= 1
+        if last == 0:
+            last = n_passes - 1
     def dead(j):
-        return 0 < j < n_passes - 1 and j not in varying_bytes
+        return j > last or (0 < j < last and j not in varying_bytes)
     parity = sum(dead(j) for j in range(1, pass_no)) & 1
     nxt = pass_no + 1
-    while dead(nxt):
+    while nxt < last and dead(nxt):
         nxt += 1
     prv = pass_no - 1
-    while dead(prv):
+    while prv > 0 and dead(prv):
         prv -= 1
-    return dead(pass_no), parity, nxt, prv
+    return dead(pass_no), parity, nxt, prv, pass_no == last
 
 
 def input_buffer(pass_no, parity):
     return ((pass_no - 1) & 1) ^ parity
 
 
+@pytest.mark.parametrize("early_last", [False, True])
 @pytest.mark.parametrize("n_passes", [3, 4, 8, 16])
-def test_every_set_of_dead_passes(n_passes):
-    middle = list(range(1, n_passes - 1))
-    subsets = itertools.chain.from_iterable(itertools.combinations(middle, k) for k in range(len(middle) + 1))
-    if n_passes == 16:   # 2^14 subsets: a spread of them
+def test_every_set_of_dead_passes(n_passes, early_last):
+    """Bytes 1 .. n-1 constant in every combination (byte 0 is never looked at: pass 0 always
+    runs).  Without early_last the top pass runs whatever its byte does."""
+    others = list(range(1, n_passes))
+    subsets = itertools.chain.from_iterable(itertools.combinations(others, k) for k in range(len(others) + 1))
+    if n_passes == 16:   # 2^15 subsets: a spread of them
         subsets = (s for i, s in enumerate(subsets) if i % 37 == 0)
-    for dead_set in subsets:
-        varying = set(range(n_passes)) - set(dead_set)
+    for constant in subsets:
+        varying = set(range(n_passes)) - set(constant)
+        live_after_0 = [j for j in range(1, n_passes) if j in varying]
+        if early_last and live_after_0:
+            writer = live_after_0[-1]
+        else:
+            writer = n_passes - 1
+        runs = {0, writer} | {j for j in live_after_0 if j < writer}
         holder = "input"          # where the data is
         side_for = None           # which pass the side-band in memory is for
         flag_owner = [None, None]  # which pass wrote each flag slot last
         last_live = None
         for k in range(n_passes):
-            skip, parity, nxt, prv = plan(varying, k, n_passes)
-            assert skip == (k in dead_set)
+            skip, parity, nxt, prv, is_last = plan(varying, k, n_passes, early_last)
+            assert skip == (k not in runs), (constant, k)
+            assert is_last == (k == writer)
             if skip:
                 continue          # moves nothing, writes no side-band and no flag
-            first, last = k == 0, k == n_passes - 1
+            first = k == 0
             if not first:
                 assert prv == last_live
-                assert holder == input_buffer(k, parity), (dead_set, k)
+                assert holder == input_buffer(k, parity), (constant, k)
                 # the upsweep of this pass may count the side-band: it must be the one for this pass,
                 # announced in the flag slot of the pass that wrote it
-                assert side_for == k and flag_owner[prv & 1] == prv, (dead_set, k)
-            if last:
+                assert side_for == k and flag_owner[prv & 1] == prv, (constant, k)
+            if is_last:
                 holder = "output"
             else:
                 out = input_buffer(k, parity) ^ 1
@@ -61,6 +77,6 @@ def test_every_set_of_dead_passes(n_passes):
                 holder = out
                 side_for = nxt
                 flag_owner[k & 1] = k
-                assert nxt > k and (nxt == n_passes - 1 or nxt not in dead_set)
+                assert nxt > k and nxt in runs
             last_live = k
         assert holder == "output"
