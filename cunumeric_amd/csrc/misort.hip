@@ -258,7 +258,7 @@ struct Plan {
   // byte carry, only where few digit values are in use; it says so per row in side_flag
   bool side_adaptive = false;
   size_t off_digits = 0, off_side_flag = 0;
-  // middle passes whose digit is the same in every key are skipped (decided on the device from
+  // passes after the first whose digit is the same in every key are skipped (decided on the device from
   // the OR of the keys and of their complements, which the first upsweep leaves in key_bits)
   bool skip_dead_passes = false;
   bool early_last = false;  // the last pass whose digit varies writes the result (large sorts only)

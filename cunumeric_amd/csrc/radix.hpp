@@ -69,7 +69,7 @@ struct PassParams {
   // device: the first upsweep ORs all keys and all complemented keys into key_bits_out
   // (KEY_BITS_SLOTS copies of {or lo, or hi, or-of-complement lo, hi}); a bit varies iff it
   // is set in both.  Every later
-  // kernel reads the four words (key_bits) and works out for itself which middle passes are
+  // kernel reads the four words (key_bits) and works out for itself which passes are
   // dead, hence which of the two ping-pong buffers holds its input (key_buf / pay_buf; the
   // keys_in .. pay_out above are what they would be with no pass skipped), and which pass is
   // the next live one (whose digit the side-band carries).  NULL: no pass is skipped.
@@ -302,8 +302,9 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
     const PassPlan plan = plan_pass(p);
     if (plan.skip) return;  // every key has the same digit: the scatter of this pass is skipped too
     if (plan.const_digit >= 0) {
-      // the last pass, which always runs, over a digit that no key varies in: the counts are
-      // the lengths of the chunks, no key needs to be read
+      // a pass that runs over a digit that no key varies in (the pass over the most
+      // significant digit where it is not left out): the counts are the lengths of the
+      // chunks, no key needs to be read
       const uint64_t clen = (uint64_t)p.tiles_per_chunk * p.tile, b0 = (uint64_t)chunk * clen;
       const uint64_t b1   = b0 + clen < p.row_len ? b0 + clen : p.row_len;
       const uint32_t cnt  = b1 > b0 ? (uint32_t)(b1 - b0) : 0u;
