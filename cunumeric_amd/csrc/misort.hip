@@ -261,7 +261,9 @@ struct Plan {
   // passes after the first whose digit is the same in every key are skipped (decided on the device from
   // the OR of the keys and of their complements, which the first upsweep leaves in key_bits)
   bool skip_dead_passes = false;
-  bool early_last = false;  // the last pass whose digit varies writes the result (large sorts only)
+  // > 0: the last pass whose digit varies writes the result if it is one of passes 1 .. this
+  // (large sorts only)
+  int early_last = 0;
   size_t off_key_bits = 0;
   size_t off_gather_idx = 0, off_gather_src = 0;
   // counting sort of 2-byte keys: chunks of the histogram kernel, counters, their scan
@@ -402,7 +404,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // two buffers the last pass leaves free)
     pl.skip_dead_passes = skip_passes_default() && pl.n_passes >= 3 && !pl.specials;
     // (one more launch per middle pass, about 5 us each: from 256 MB of keys on)
-    pl.early_last = pl.skip_dead_passes && pl.volume * pl.dt.bytes >= early_last_min_bytes();
+    pl.early_last =
+      (pl.skip_dead_passes && pl.volume * pl.dt.bytes >= early_last_min_bytes()) ? (int)pl.n_passes / 2 : 0;
     pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
     pl.side_adaptive = side_band_default() && !pl.side_band && pl.n_passes >= 2 && pl.dt.bytes >= 4 &&
                        (pl.pay != PAY_NONE || pl.dt.bytes > 4);
@@ -634,14 +637,14 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
       unsigned long long* bits = reinterpret_cast<unsigned long long*>(S + pl.off_key_bits);
       pp.key_bits_out = (pl.skip_dead_passes && first) ? bits : nullptr;
       pp.key_bits     = pl.skip_dead_passes ? bits : nullptr;  // complete once the first upsweep has run
-      pp.early_last   = pl.early_last ? 1 : 0;
+      pp.early_last   = pl.early_last;
     }
     pp.slab_tot = reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + (pass & 1) * pl.slab_tot_bytes);
     pp.slab_tot_next =
       last ? nullptr
            : reinterpret_cast<unsigned long long*>(S + pl.off_slab_tot + ((pass + 1) & 1) * pl.slab_tot_bytes);
     launch_pass<KeyT, PAY>(L, pl, first, last, pp);
-    if (pl.early_last && !first && !last) {
+    if (pass >= 1 && pass <= pl.early_last && !last) {
       // If no key varies in any digit after this one, this pass writes the result: the same
       // scatter in its last-pass form, which returns at once otherwise (as the form above
       // does in that case).

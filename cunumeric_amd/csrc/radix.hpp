@@ -33,6 +33,8 @@
 #include <stdint.h>
 
 #include "keyspec.hpp"
+#include <type_traits>
+
 #include "lanes.hpp"
 
 namespace misort {
@@ -77,7 +79,9 @@ struct PassParams {
   unsigned long long* key_bits_out;
   void* key_buf[2];
   void* pay_buf[2];
-  int early_last;  // leading digits that no key varies in are left out too: see plan_pass
+  int early_last;  // > 0: the highest pass that may write the result in place of the pass over the
+                   // most significant digit (see plan_pass); the host launches the scatter of
+                   // passes 1 .. early_last in both forms
   const void* pay_in;    // PAY_IDX32: u32 (ignored when FIRST); PAY_I64: int64, NULL => positions
   void* pay_out;         // PAY_IDX32: u32, int64 when LAST; PAY_I64: int64
   uint32_t* chunk_hist;             // [rows * chunks_per_row][RADIX] counts of this pass
@@ -114,9 +118,10 @@ struct PassPlan {
 // Pass 0 transforms the elements into keys and is never skipped.  The pass over the most
 // significant digit transforms them back: without early_last it always runs (and skips the
 // counting if its digit is constant); with early_last the last pass whose digit varies
-// writes the result instead (the host launches, for every pass after the first, the scatter
-// kernel in both forms, and each finds out here whether it is the one to run), unless that
-// would be pass 0, which cannot be first and last at once when it sorts in place.
+// writes the result instead if it is one of passes 1 .. early_last (the host launches the
+// scatter kernel of those passes in both forms, and each finds out here whether it is the one
+// to run; pass 0 cannot be first and last at once when it sorts in place, and a pass in the
+// upper half would save little for one more launch per pass).
 __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
 {
   PassPlan r{false, p.pass == p.n_passes - 1, 0u, p.shift + RADIX_BITS, p.pass - 1, -1};
@@ -134,15 +139,21 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
   }
   const unsigned long long lo = uniform64(w[0] & w[2]);
   const unsigned long long hi = uniform64(w[1] & w[3]);
-  auto constant = [&](int j) {  // no key varies in digit j
-    const unsigned long long w = j < 8 ? lo : hi;
+  // Signed integers (at most 8 bytes: the second pair of words is free for them): a digit
+  // below the most significant one that only repeats the sign in every key (small values of
+  // both signs: 0x00 / 0xFF) needs no pass either, since the pass over the most significant
+  // digit, which then runs because the sign varies, puts the signs apart; the words say that
+  // of the values with their sign extension taken out.
+  const bool by_magnitude = p.xform == XF_SIGNED && p.n_passes <= 8;
+  auto constant = [&](int j) {  // no key varies in digit j (or only with the sign)
+    const unsigned long long w = (by_magnitude && j < p.n_passes - 1) ? hi : (j < 8 ? lo : hi);
     return ((w >> (8 * (j & 7))) & 0xFFull) == 0;
   };
   // the last pass that runs
   int last = p.n_passes - 1;
   if (p.early_last) {
     while (last > 0 && constant(last)) --last;
-    if (last == 0) last = p.n_passes - 1;
+    if (last == 0 || last > p.early_last) last = p.n_passes - 1;
   }
   auto dead = [&](int j) { return j > last || (j > 0 && j < last && constant(j)); };
   for (int j = 1; j < p.pass; ++j) r.parity ^= dead(j) ? 1u : 0u;
@@ -155,9 +166,12 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
   while (pv > 0 && dead(pv)) --pv;
   r.prev_live = pv;
   {
+    // (a pass that runs over a constant digit is the one over the most significant digit,
+    // which the words of the keys themselves describe)
     const unsigned long long ones = uniform64(p.pass < 8 ? w[0] : w[1]);
     const int sh = 8 * (p.pass & 7);
-    if (constant(p.pass)) r.const_digit = (int)((ones >> sh) & 0xFFull);
+    if (constant(p.pass) && !(by_magnitude && p.pass < p.n_passes - 1))
+      r.const_digit = (int)((ones >> sh) & 0xFFull);
   }
   return r;
 }
@@ -358,6 +372,15 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       } else {
         or_lo |= (unsigned long long)k;
         nor_lo |= (unsigned long long)(KeyT)~k;
+        if (p.xform == XF_SIGNED) {
+          // signed integers: the same for the value with its sign extension taken out
+          // (x ^ (x >> all), i.e. x or ~x): bytes that only repeat the sign come out zero
+          using S      = typename std::make_signed<KeyT>::type;
+          const KeyT x = (KeyT)(k ^ (KeyT)((KeyT)1 << (sizeof(KeyT) * 8 - 1)));
+          const KeyT t = (KeyT)(x ^ (KeyT)((S)x >> (sizeof(KeyT) * 8 - 1)));
+          or_hi |= (unsigned long long)t;
+          nor_hi |= (unsigned long long)(KeyT)~t;
+        }
       }
     }
     atomicAdd(&my[KeyOps<KeyT>::digit(k, p.shift) * COPIES], 1u);
@@ -419,7 +442,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       for (int s = 32; s > 0; s >>= 1) {
         or_lo |= __shfl_xor(or_lo, s, 64);
         nor_lo |= __shfl_xor(nor_lo, s, 64);
-        if (sizeof(KeyT) == 16) {
+        if (sizeof(KeyT) == 16 || p.xform == XF_SIGNED) {
           or_hi |= __shfl_xor(or_hi, s, 64);
           nor_hi |= __shfl_xor(nor_hi, s, 64);
         }
@@ -436,7 +459,8 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   if constexpr (FIRST) {
     // Atomics on one address queue up (about 10 ns each), so a workgroup adds its bits once,
     // to one of KEY_BITS_SLOTS copies of the words, and nobody waits for the result.
-    if (p.key_bits_out && threadIdx.x < 4 && (sizeof(KeyT) == 16 || (threadIdx.x & 1) == 0)) {
+    if (p.key_bits_out && threadIdx.x < 4 &&
+        (sizeof(KeyT) == 16 || p.xform == XF_SIGNED || (threadIdx.x & 1) == 0)) {
       unsigned long long v = 0;
 #pragma unroll
       for (int w = 0; w < NW; ++w) v |= wg_bits[w * 4 + threadIdx.x];

@@ -3,7 +3,9 @@ partition / argpartition (the contract), misort_select (elements kth, kth + 1 an
 stable sort), sort (bit-exact) and stable argsort (exact), over element types, row counts,
 row lengths off every alignment and key distributions that steer the kernels differently:
 full range, few values, pools of repeated values (runs of equal keys in the later passes),
-small ranges (dead leading bytes), sorted input, one value holding most of the row."""
+small ranges (dead leading bytes), sorted input, one value holding most of the row, small values
+of both signs.  Half of the seeds also let small sorts leave out constant leading digits
+(MISORT_EARLY_LAST_BYTES=0), which large sorts do by themselves."""
 import numpy as np
 import pytest
 
@@ -32,14 +34,23 @@ def draw(rng, dtype, rows, n, kind):
         a = np.sort(random_array(dtype, total, rng, specials=False))
         if rng.integers(0, 2):
             a = a[::-1].copy()
-    else:
+    elif kind == 5:
         a = random_array(dtype, total, rng, specials=False)
         a[rng.random(total) < 0.7] = a[0]
+    else:
+        r = int(rng.choice([1, 100, 40000, 1 << 20]))
+        off = int(rng.choice([0, 0, -r, 1 << 28, -(1 << 29)]))
+        a = rng.integers(-r, r, total, endpoint=True) + off
+        a = np.abs(a).astype(dtype) if np.dtype(dtype).kind == "u" else a.astype(dtype)
     return np.ascontiguousarray(a).reshape(rows, n)
 
 
 @pytest.mark.parametrize("seed", range(6))
-def test_random_cases(seed):
+def test_random_cases(seed, monkeypatch):
+    if seed % 2:
+        monkeypatch.setenv("MISORT_EARLY_LAST_BYTES", "0")
+    else:
+        monkeypatch.delenv("MISORT_EARLY_LAST_BYTES", raising=False)
     abi = Abi()
     rng = np.random.default_rng(1000 + seed)
     for it in range(12):
@@ -47,7 +58,7 @@ def test_random_cases(seed):
         rows = int(rng.choice([1, 1, 2, 3, 7, 20]))
         n = int(rng.choice([65536, 65537, 70001, 100003, 131072, 200001, 262144 + 5, 500009]))
         rows = min(rows, max(1, 3_000_000 // n))
-        kind = int(rng.integers(0, 6))
+        kind = int(rng.integers(0, 7))
         a = draw(rng, dtype, rows, n, kind)
         kth = int(rng.choice([0, 1, n // 2, n - 2, n - 1, int(rng.integers(0, n))]))
         tag = f"seed={seed} it={it} dtype={np.dtype(dtype).name} rows={rows} n={n} kind={kind} kth={kth}"

@@ -89,6 +89,30 @@ def test_small_ranges_rows_and_payload(abi, dtype, early_last):
     assert bits_equal(got, np.sort(flat[:row_len], kind="stable"))
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.int64], ids=lambda d: np.dtype(d).name)
+def test_small_values_of_both_signs(abi, dtype, early_last):
+    """Signed integers near zero: the upper bytes only repeat the sign (0x00 / 0xFF), which
+    the pass over the most significant byte sorts out, so the passes over them are left out
+    although their digits differ between keys."""
+    rng = np.random.default_rng(65)
+    ii = np.iinfo(dtype)
+    n = 250007
+    ranges = [(-1000, 1000), (-70000, 5), (-1, 0), (-50000, -1), (-3, 300), (ii.min, ii.min + 1000),
+              (ii.max - 5, ii.max), (-(1 << (ii.bits - 9)), 1 << (ii.bits - 9))]
+    for lo, hi in ranges:
+        a = rng.integers(lo, hi, n, dtype=dtype, endpoint=True)
+        print(f"skip passes signed dtype={np.dtype(dtype).name} range=({lo}, {hi})", flush=True)
+        assert np.array_equal(abi.local_sort(a, n, argsort=False), np.sort(a)), (lo, hi)
+        assert np.array_equal(abi.local_sort(a, n, argsort=True, chunks=5), np.argsort(a, kind="stable")), (lo, hi)
+    # a few far-off values among small ones, rows, and the extremes
+    a = rng.integers(-500, 500, 3 * 100003, dtype=dtype)
+    a[rng.integers(0, a.size, 7)] = [ii.min, ii.max, ii.min + 1, -1, 0, ii.max - 1, 1 << (ii.bits - 2)]
+    a = a.reshape(3, 100003)
+    got = abi.local_sort(a, 100003, argsort=True).reshape(3, -1)
+    assert np.array_equal(got, np.argsort(a, axis=1, kind="stable"))
+    assert np.array_equal(abi.local_sort(a, 100003, argsort=False).reshape(3, -1), np.sort(a, axis=1))
+
+
 def test_large_int64_small_range(abi, early_last):
     rng = np.random.default_rng(63)
     n = 1 << 24
