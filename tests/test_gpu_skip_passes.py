@@ -54,7 +54,8 @@ WIDTH8 = [(0,), (0, 1), (0, 7), (3, 4), (7,), (1, 2, 3, 4, 5, 6), (0, 2, 4, 6), 
 def test_constant_bytes_in_every_position(abi, dtype, patterns, early_last):
     rng = np.random.default_rng(61)
     n = 300007
-    assert ("early_last=1" in abi.describe_plan(dtype, n, n, True)) == early_last
+    if os.environ.get("MISORT_SKIP_PASSES") != "0":
+        assert ("early_last=1" in abi.describe_plan(dtype, n, n, True)) == early_last
     for live in patterns:
         a = masked_random(dtype, n, rng, live)
         for chunks in (0, 3):
@@ -120,7 +121,8 @@ def test_large_int64_small_range(abi, early_last):
     print("skip passes int64 2^24 values below 50000", flush=True)
     assert np.array_equal(abi.local_sort(a, n, argsort=True), np.argsort(a, kind="stable"))
     assert np.array_equal(abi.local_sort(a, n, argsort=False), np.sort(a))
-    assert "skip_dead_passes=1" in abi.describe_plan(np.int64, n, n, True)
+    if os.environ.get("MISORT_SKIP_PASSES") != "0":
+        assert "skip_dead_passes=1" in abi.describe_plan(np.int64, n, n, True)
 
 
 def test_switch_off_gives_the_same_result():
