@@ -545,11 +545,22 @@ static void launch_zero(Launcher& L, void* p, size_t bytes)
 }
 
 template <typename KeyT, int PAY>
-static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
+static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
 {
   const size_t eb    = sizeof(KeyT);
   const char* vin    = reinterpret_cast<const char*>(a.values_in);
   char* vout         = reinterpret_cast<char*>(a.values_out);
+  // Keys-only float sorts restore the bit patterns of their zeros and NaNs afterwards.  In
+  // place, those are set aside before the last pass overwrites the input, in the ping-pong
+  // buffer that pass leaves free, which is known on the host only if every pass runs.  Out
+  // of place the input outlives the sort, they are taken from there at the end, and passes
+  // may be skipped as in every other sort.
+  Plan pl                  = plan;
+  const bool specials_late = pl.specials && vin != vout;
+  if (specials_late && skip_passes_default() && pl.n_passes >= 3) {
+    pl.skip_dead_passes = true;
+    pl.early_last = pl.volume * pl.dt.bytes >= early_last_min_bytes() ? (int)pl.n_passes / 2 : 0;
+  }
   const int64_t* iin = a.indices_in;
   int64_t* iout      = a.indices_out;
   char* S            = a.scratch;
@@ -665,7 +676,7 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
                              (uint32_t)(pl.chunks_per_row * (kUpsweepThreads / 64)));
         });
       }
-      if (pl.specials && pass == pl.n_passes - 2) {
+      if (pl.specials && !specials_late && pass == pl.n_passes - 2) {
         // The buffer the last pass will not read is free now, and the input is still intact
         // (only the last pass writes values_out, which may alias values_in): collect the
         // original zeros / NaNs there, in input order.
@@ -675,7 +686,7 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
                              dim3((unsigned)pl.n_chunks), dim3(kUpsweepThreads), 0, L.stream,
                              reinterpret_cast<const KeyT*>(vin), side, special_blk, special_row,
                              (uint64_t)pl.row_len, (uint32_t)pl.chunks_per_row,
-                             (uint64_t)pl.tiles_per_chunk * pl.tile);
+                             (uint64_t)pl.tiles_per_chunk * pl.tile, false);
         });
       }
     }
@@ -687,7 +698,14 @@ static void radix_sort_rows(Launcher& L, const Plan& pl, const SortArgs& a)
   if (alias_pay) launch_copy(L, K_COPY, iout, S + pl.off_pay[0], pl.volume * pay_bytes);
 
   if constexpr (is_float_width<KeyT>() && PAY == PAY_NONE) {
-    if (pl.specials) {
+    if (specials_late) {
+      L.run(K_SPECIAL_COLLECT, [&] {
+        hipLaunchKernelGGL((special_collect_kernel<KeyT, kUpsweepThreads>), dim3((unsigned)pl.n_chunks),
+                           dim3(kUpsweepThreads), 0, L.stream, reinterpret_cast<const KeyT*>(vin),
+                           reinterpret_cast<KeyT*>(vout), special_blk, special_row, (uint64_t)pl.row_len,
+                           (uint32_t)pl.chunks_per_row, (uint64_t)pl.tiles_per_chunk * pl.tile, true);
+      });
+    } else if (pl.specials) {
       const KeyT* side = reinterpret_cast<const KeyT*>(S + pl.off_keys[(pl.n_passes - 1) & 1]);
       size_t bpr       = (pl.row_len + 16383) / 16384;
       if (bpr > 1024) bpr = 1024;
@@ -762,7 +780,7 @@ static void count16_sort(Launcher& L, const Plan& pl, const SortArgs& a)
     L.run(K_SPECIAL_COLLECT, [&] {
       hipLaunchKernelGGL((special_collect_kernel<uint16_t, C16_HIST_NT>), dim3((unsigned)pl.c16_chunks),
                          dim3(C16_HIST_NT), 0, L.stream, vin, side, special_blk, special_row, n,
-                         (uint32_t)pl.c16_chunks, (uint64_t)pl.c16_chunk_len);
+                         (uint32_t)pl.c16_chunks, (uint64_t)pl.c16_chunk_len, false);
     });
   }
   constexpr uint64_t span = (uint64_t)C16_FILL_NT * C16_FILL_VEC * 8;

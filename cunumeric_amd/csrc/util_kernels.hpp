@@ -219,13 +219,16 @@ special_scan_kernel(unsigned long long* blk, const unsigned long long* rowctr,
   }
 }
 
-// same grid and wave sub-chunk ownership as the first upsweep
+// same grid and wave sub-chunk ownership as the first upsweep.  into_sorted: `side` is the
+// sorted output itself (the input is a different buffer and still intact after the sort):
+// the zeros go straight over its zero run, which starts behind the negatives, the NaNs over
+// its tail, and no patch kernel follows.
 template <typename KeyT, int NT>
 __global__ void __launch_bounds__(NT)
 special_collect_kernel(const KeyT* __restrict__ in, KeyT* __restrict__ side,
                        const unsigned long long* __restrict__ blk,
                        const unsigned long long* __restrict__ rowctr, uint64_t row_len,
-                       uint32_t chunks_per_row, uint64_t chunk)
+                       uint32_t chunks_per_row, uint64_t chunk, bool into_sorted)
 {
   constexpr int NW          = NT / 64;
   const uint32_t row        = blockIdx.x / chunks_per_row;
@@ -240,7 +243,7 @@ special_collect_kernel(const KeyT* __restrict__ in, KeyT* __restrict__ side,
   uint64_t end         = begin + sub;
   if (end > row_len) end = row_len;
   const uint64_t e     = ((uint64_t)row * chunks_per_row + c) * NW + wave;
-  unsigned long long zoff = blk[2 * e];
+  unsigned long long zoff = blk[2 * e] + (into_sorted ? ctr[SP_NEG] : 0ull);
   unsigned long long noff = row_len - ctr[SP_NAN] + blk[2 * e + 1];
   const KeyT* rin = in + (uint64_t)row * row_len;
   KeyT* rside     = side + (uint64_t)row * row_len;

@@ -114,6 +114,33 @@ def test_small_values_of_both_signs(abi, dtype, early_last):
     assert np.array_equal(abi.local_sort(a, 100003, argsort=False).reshape(3, -1), np.sort(a, axis=1))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=lambda d: np.dtype(d).name)
+def test_float_values_with_constant_mantissa_bytes(abi, dtype, early_last):
+    """Keys-only float sorts out of place: integer-valued floats have constant low mantissa
+    bytes, whose passes are skipped; the zeros of both signs and the NaNs (with their
+    payloads) are restored from the input after the sort.  In place every pass runs (the
+    zeros and NaNs are set aside before the last one); both must give NumPy's bits."""
+    rng = np.random.default_rng(66)
+    rows, n = 2, 150001
+    for hi in (200, 60000, 1 << 22):
+        a = rng.integers(-hi, hi, rows * n).astype(dtype)
+        u = a.view(np.dtype(f"u{a.dtype.itemsize}"))
+        where = rng.integers(0, a.size, a.size // 50)
+        a[where[: where.size // 3]] = -0.0
+        a[where[where.size // 3: 2 * where.size // 3]] = 0.0
+        nan_bits = (np.array(np.nan, dtype=dtype).view(u.dtype) | rng.integers(1, 1000, where.size).astype(u.dtype))
+        u[where[2 * where.size // 3:]] = nan_bits[2 * where.size // 3:]
+        a = a.reshape(rows, n)
+        ref = np.sort(a, axis=1, kind="stable")
+        print(f"skip passes float values dtype={np.dtype(dtype).name} below {hi}", flush=True)
+        got = abi.local_sort(a, n, argsort=False).reshape(rows, n)
+        assert bits_equal(got, ref), hi
+        got = abi.local_sort(a, n, argsort=False, chunks=7).reshape(rows, n)
+        assert bits_equal(got, ref), hi
+        got = abi.local_sort(a, n, argsort=False, inplace=True).reshape(rows, n)
+        assert bits_equal(got, ref), hi
+
+
 def test_large_int64_small_range(abi, early_last):
     rng = np.random.default_rng(63)
     n = 1 << 24
