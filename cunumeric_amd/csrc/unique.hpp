@@ -216,8 +216,11 @@ unique_compact_kernel(const Raw* __restrict__ s, uint64_t n, int xform,
     }
   } else {
     // thread t owns the consecutive elements base + t * IPT ..: run heads keep their order
-    constexpr uint64_t IPT = BLK / UNIQ_NT;
-    const uint64_t mine    = base + (uint64_t)threadIdx.x * IPT;
+    // (IPT from what the block holds: a short array is spread over all threads instead of
+    // walked by the first few, element after element)
+    const uint64_t left = n - base < BLK ? n - base : BLK;
+    const uint64_t IPT  = (left + UNIQ_NT - 1) / UNIQ_NT;
+    const uint64_t mine = base + (uint64_t)threadIdx.x * IPT;
     uint32_t c = 0;
     for (uint64_t i = mine; i < mine + IPT && i < n; ++i) c += unique_is_head(s, i, xform);
     __shared__ uint32_t wsum[NW];
