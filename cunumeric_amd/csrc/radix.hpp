@@ -415,7 +415,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   const KeyT* base  = in + begin;
   auto count_all = [&](auto sw) {
     uint64_t done = 0;
-    if (V > 1 && (reinterpret_cast<uintptr_t>(base) & 15) == 0) {
+    if (sizeof(Vec) == 16 && (reinterpret_cast<uintptr_t>(base) & 15) == 0) {  // (16-byte keys: one per load)
       constexpr int U     = 4;
       const uint64_t nvec = n / V;
       const Vec* vbase    = reinterpret_cast<const Vec*>(base);
