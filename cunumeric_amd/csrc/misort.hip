@@ -238,6 +238,10 @@ struct Plan {
   size_t volume = 0, row_len = 0, rows = 0;
   bool argsort = false, has_indices_in = false;
   bool gather_values = false;  // complex keys-only: argsort, then gather the elements
+  // complex64 keys-only on the radix path: the elements travel through the passes as an 8-byte
+  // payload instead (4 bytes more per key and pass than a position, but no gather at the end:
+  // 2^26 elements 5.46 -> 4.92 ms)
+  bool values_as_payload = false;
   int pay = PAY_NONE;
   int n_passes = 0;
   int tile = 0;
@@ -341,6 +345,13 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.strategy = S_COUNT8;  // any single row too long for the row kernels
   } else {
     pl.strategy = S_RADIX;
+  }
+  if (pl.strategy == S_RADIX && pl.gather_values && pl.dt.bytes == 8) {
+    pl.gather_values     = false;
+    pl.values_as_payload = true;
+    pl.pay               = PAY_I64;
+    pl.argsort           = true;
+    pl.has_indices_in    = true;
   }
 
   size_t off = 0;
@@ -1037,6 +1048,11 @@ static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_
   // (canonical_values: the caller only compares the sorted values through their keys, so the
   // last pass may write them through the inverse key transform, which maps -0 to +0 and
   // every NaN to one NaN; not for complex elements, whose NaN tiers have no inverse)
+  if (pl.values_as_payload) {  // the elements are the payload of their own keys
+    core.indices_in  = reinterpret_cast<const int64_t*>(values_in);
+    core.indices_out = reinterpret_cast<int64_t*>(values_out);
+    core.values_out  = nullptr;
+  }
   const bool gather_sorted =
     argsort && values_out && !indices_in && !(canonical_values && pl.dt.xform != XF_COMPLEX);
   if (gather_sorted) core.values_out = nullptr;
