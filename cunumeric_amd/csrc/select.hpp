@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
     // 16-byte loads where the row allows it; in whole batches only when appending, so that the
     // rest is done with the wavefronts intact
     uint64_t i0 = b0;
-    if (V > 1 && (reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
+    if (sizeof(Vec) == 16 && (reinterpret_cast<uintptr_t>(base + b0) & 15) == 0) {
       uint64_t nvec = (b1 - b0) / V;
       if (ST == SEL_APPEND) nvec -= nvec % ((uint64_t)SEL_NT * U);
       const Vec* vb = reinterpret_cast<const Vec*>(base + b0);
