@@ -393,13 +393,23 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       }
     }
     atomicAdd(&my[KeyOps<KeyT>::digit(k, p.shift) * COPIES], 1u);
+  };
+  // SPECIALS: zeros, NaNs, negative zeros, and the elements that sort before the zeros
+  // (sign set, neither zero nor NaN: counted as sign bits minus the negative zeros and NaNs).
+  // Zeros and NaNs are rare, so a whole 16-byte load is asked at once whether it holds any
+  // (smallest and largest of the values without their signs), and looked at one by one only then.
+  uint32_t n_sign = 0, n_negnan = 0;
+  constexpr int KEY_BITS = (int)sizeof(KeyT) * 8;
+  auto special_one = [&](KeyT raw) {
     if constexpr (SPECIALS) {
-      using F = FloatBits<KeyT>;
-      const bool isn = float_is_nan(raw);
+      using F         = FloatBits<KeyT>;
+      const bool isn  = float_is_nan(raw);
+      const bool isz  = (KeyT)(raw & (KeyT)~F::SIGN) == 0;
+      const bool sign = (raw & F::SIGN) != 0;
       n_nan += isn;
-      n_zero += (KeyT)(raw & (KeyT)~F::SIGN) == 0;
-      n_negzero += raw == F::SIGN;
-      n_neg += !isn && (raw & F::SIGN) != 0 && raw != F::SIGN;  // sorts before the zeros
+      n_zero += isz;
+      n_negzero += isz && sign;
+      n_negnan += isn && sign;
     }
   };
 
@@ -422,15 +432,38 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       stream_vectors<U>(vbase, nvec, first, width, [&](const Vec& r) {
 #pragma unroll
         for (int e = 0; e < V; ++e) count(r.v[e], sw);
+        if constexpr (SPECIALS && sizeof(KeyT) <= 8) {
+          using F = FloatBits<KeyT>;
+          KeyT least = (KeyT)~(KeyT)0, most = 0;
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            const KeyT t = (KeyT)(r.v[e] << 1);  // without the sign
+            least        = t < least ? t : least;
+            most         = t > most ? t : most;
+            n_sign += (uint32_t)(r.v[e] >> (KEY_BITS - 1));
+          }
+          if (least == 0 || most > (KeyT)(F::EXP << 1)) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) special_one(r.v[e]);
+          }
+        }
       });
       done = nvec * V;
     }
-    for (uint64_t i = done + first; i < n; i += width) count(base[i], sw);
+    for (uint64_t i = done + first; i < n; i += width) {
+      const KeyT raw = base[i];
+      count(raw, sw);
+      if constexpr (SPECIALS && sizeof(KeyT) <= 8) {
+        n_sign += (uint32_t)(raw >> (KEY_BITS - 1));
+        special_one(raw);
+      }
+    }
   };
   if (FIRST && sizeof(KeyT) <= 8 && p.key_bits_out && p.xform == XF_SIGNED) count_all(std::true_type{});
   else count_all(std::false_type{});
 
   if constexpr (SPECIALS) {
+    n_neg = n_sign - n_negzero - n_negnan;
 #pragma unroll
     for (int s = 32; s > 0; s >>= 1) {
       n_zero += __shfl_xor(n_zero, s, 64);
