@@ -368,10 +368,11 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   uint32_t n_zero = 0, n_nan = 0, n_negzero = 0, n_neg = 0;
   // FIRST: OR of the keys and of their complements (which bits vary over the whole input)
   unsigned long long or_lo = 0, or_hi = 0, nor_lo = 0, nor_hi = 0;
-  // (sw: the words of signed integers are wanted too; decided once, outside the loop: with
+  // (sw = 1: the words of signed integers are wanted too; decided once, outside the loop: with
   // the test inside it the first upsweep of every other type ran 7 % longer)
   auto count = [&](KeyT raw, auto sw) {
-    const KeyT k = FIRST ? KeyOps<KeyT>::to_key(raw, p.xform) : raw;
+    // (mode 2: the transform is known to be the complex one, so its test leaves the loop too)
+    const KeyT k = FIRST ? KeyOps<KeyT>::to_key(raw, decltype(sw)::value == 2 ? (int)XF_COMPLEX : p.xform) : raw;
     if constexpr (FIRST) {
       if constexpr (sizeof(KeyT) == 16) {
         or_lo |= k.lo;
@@ -381,7 +382,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       } else {
         or_lo |= (unsigned long long)k;
         nor_lo |= (unsigned long long)(KeyT)~k;
-        if constexpr (decltype(sw)::value) {
+        if constexpr (decltype(sw)::value == 1) {
           // signed integers: the same for the value with its sign extension taken out
           // (x ^ (x >> all), i.e. x or ~x): bytes that only repeat the sign come out zero
           using S      = typename std::make_signed<KeyT>::type;
@@ -459,8 +460,12 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
       }
     }
   };
-  if (FIRST && sizeof(KeyT) <= 8 && p.key_bits_out && p.xform == XF_SIGNED) count_all(std::true_type{});
-  else count_all(std::false_type{});
+  if (FIRST && sizeof(KeyT) <= 8 && p.key_bits_out && p.xform == XF_SIGNED)
+    count_all(std::integral_constant<int, 1>{});
+  else if (FIRST && sizeof(KeyT) == 8 && p.xform == XF_COMPLEX)
+    count_all(std::integral_constant<int, 2>{});
+  else
+    count_all(std::integral_constant<int, 0>{});
 
   if constexpr (SPECIALS) {
     n_neg = n_sign - n_negzero - n_negnan;
