@@ -388,7 +388,7 @@ def run_partition(args) -> int:
         "vs_baseline": None, "dtype": "u32", "data": "synthetic",
         "config": {"workload": f"argpartition, float32 (C2 input), n=2^{log2n}, kth=n/2, int64 positions"},
         "parity_guard": "ok" if ok else "FAILED",
-        "roofline": {"bound": "hbm", "kernel": "select_hist + split_downsweep", "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "select_hist + select_split", "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "achieved": b * n / dt / 1e9, "frac": b * n / dt / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "note": "whole call, 20 algorithmic bytes per key"},
         "cpu_baseline": {"value": cpu, "unit": "Gkeys/s", "cores": 1, "kind": "port",

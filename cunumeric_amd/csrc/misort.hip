@@ -121,7 +121,7 @@ static const char* const kKernelNames[K_NUM] = {
   "count16_hist",    "count16_scan",    "count16_fill",     "searchsorted",
   "unique_count",    "unique_offsets",  "unique_compact",   "count8_hist",
   "count8_fill",     "select_init",     "select_hist",      "select_pick",
-  "select_counts",   "select_above",    "select_emit",    "split_downsweep",
+  "select_counts",   "select_above",    "select_emit",    "select_split",
   "colsort_wave"};
 
 // ---------------------------------------------------------------------------------------
