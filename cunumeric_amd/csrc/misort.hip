@@ -414,9 +414,14 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // (not for keys-only float sorts: the patch of their zeros and NaNs counts on which of the
     // two buffers the last pass leaves free)
     pl.skip_dead_passes = skip_passes_default() && pl.n_passes >= 3 && !pl.specials;
-    // (one more launch per middle pass, about 5 us each: from 256 MB of keys on)
+    // (one more launch per middle pass, about 5 us each: from 256 MB of keys on; integers
+    // only: the most significant byte of a float key holds the sign and the top of the
+    // exponent, which vary in all but contrived inputs)
     pl.early_last =
-      (pl.skip_dead_passes && pl.volume * pl.dt.bytes >= early_last_min_bytes()) ? (int)pl.n_passes / 2 : 0;
+      (pl.skip_dead_passes && (pl.dt.xform == XF_SIGNED || pl.dt.xform == XF_UNSIGNED) &&
+       pl.volume * pl.dt.bytes >= early_last_min_bytes())
+        ? (int)pl.n_passes / 2
+        : 0;
     pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
     pl.side_adaptive = side_band_default() && !pl.side_band && pl.n_passes >= 2 && pl.dt.bytes >= 4 &&
                        (pl.pay != PAY_NONE || pl.dt.bytes > 4);
@@ -570,7 +575,6 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   const bool specials_late = pl.specials && vin != vout;
   if (specials_late && skip_passes_default() && pl.n_passes >= 3) {
     pl.skip_dead_passes = true;
-    pl.early_last = pl.volume * pl.dt.bytes >= early_last_min_bytes() ? (int)pl.n_passes / 2 : 0;
   }
   const int64_t* iin = a.indices_in;
   int64_t* iout      = a.indices_out;
