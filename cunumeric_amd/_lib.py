@@ -37,6 +37,11 @@ EXPORTS = (
     "misort_select_scratch_bytes",
     "misort_select",
     "misort_sort_axis",
+    "misort_scratch_bytes_opts",
+    "misort_local_opts",
+    "misort_describe_plan_opts",
+    "misort_init",
+    "misort_rank_mode",
 )
 
 STATUS_NAMES = {
@@ -50,6 +55,16 @@ STATUS_NAMES = {
     7: "MISORT_ERR_ALIAS",
     8: "MISORT_ERR_UNSUPPORTED",
 }
+
+
+class Options(ctypes.Structure):
+    """misort_options of include/misort.h; the defaults mean "as misort_local"."""
+
+    _fields_ = [("target_chunks", c_size_t), ("early_last_min_bytes", ctypes.c_longlong),
+                ("bucket_path", c_int), ("bucket_bins", ctypes.c_uint), ("bucket_cap", ctypes.c_uint)]
+
+    def __init__(self, target_chunks=0, early_last_min_bytes=-1, bucket_path=-1, bucket_bins=0, bucket_cap=0):
+        super().__init__(target_chunks, early_last_min_bytes, bucket_path, bucket_bins, bucket_cap)
 
 
 class MisortLibraryError(RuntimeError):
@@ -138,6 +153,20 @@ def load():
         c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64,
         c_void_p, c_size_t, c_void_p, c_size_t,
     ]
+    lib.misort_scratch_bytes_opts.restype = c_size_t
+    lib.misort_scratch_bytes_opts.argtypes = [c_int, c_size_t, c_size_t, c_int, c_int, ctypes.POINTER(Options)]
+    lib.misort_local_opts.restype = c_int
+    lib.misort_local_opts.argtypes = [
+        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64,
+        c_void_p, c_size_t, c_void_p, ctypes.POINTER(Options),
+    ]
+    lib.misort_describe_plan_opts.restype = c_int
+    lib.misort_describe_plan_opts.argtypes = [c_int, c_size_t, c_size_t, c_int, c_int, ctypes.POINTER(Options),
+                                              c_char_p, c_size_t]
+    lib.misort_init.restype = c_int
+    lib.misort_init.argtypes = []
+    lib.misort_rank_mode.restype = c_int
+    lib.misort_rank_mode.argtypes = []
     lib.misort_local_static.restype = c_int
     lib.misort_local_static.argtypes = [
         c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int64, c_void_p,
@@ -159,9 +188,13 @@ def check(status: int) -> None:
 
 
 def describe_plan(dtype_code: int, volume: int, sort_dim_size: int, argsort: bool,
-                  has_indices_in: bool = False) -> str:
+                  has_indices_in: bool = False, options: "Options | None" = None) -> str:
     lib = load()
     buf = ctypes.create_string_buffer(512)
-    check(lib.misort_describe_plan(dtype_code, volume, sort_dim_size, int(argsort),
-                                   int(has_indices_in), buf, len(buf)))
+    if options is None:
+        check(lib.misort_describe_plan(dtype_code, volume, sort_dim_size, int(argsort),
+                                       int(has_indices_in), buf, len(buf)))
+    else:
+        check(lib.misort_describe_plan_opts(dtype_code, volume, sort_dim_size, int(argsort),
+                                            int(has_indices_in), ctypes.byref(options), buf, len(buf)))
     return buf.value.decode()

@@ -1,0 +1,605 @@
+// Sort of one row of a few ten thousand to about a million elements in four launches: sample
+// -> count -> scatter -> sort the bins.  It serves the sizes where the radix path's two
+// launches per digit are mostly launch and start-up time (the reference's own benchmark sorts
+// 10^6 elements, examples/sort.py:110-123; the calls replaced are the same ones,
+// src/cunumeric/sort/cub_sort.cuh:60-71, 120-143 and thrust_sort.cuh:61-66).
+//
+//   bucket_plan_kernel     one workgroup draws 16 samples per bin at scattered places, sorts
+//                          their keys in LDS and keeps every 16th as a splitter (at most 255);
+//   bucket_count_kernel    every chunk counts its keys per bin: bin 2j holds the keys strictly
+//                          between splitters j-1 and j, bin 2j+1 the keys equal to splitter j, so
+//                          a value that fills half the array fills a bin that needs no sorting;
+//   bucket_scatter_kernel  every chunk moves its elements to their bins, in input order (chunks
+//                          in order, elements of a chunk in order): the pass is stable;
+//   bucket_sort_kernel     one workgroup per bin: the bin in registers, an LSD radix sort over
+//                          the key bits that can differ inside the bin (from its two splitters),
+//                          permuting through LDS; the result goes straight to the output.
+// Splitters from a sorted sample make the bins even whatever the distribution of the keys
+// (with 16 samples per bin one four times the average is a 1e-18 event), and equal keys take no
+// room in the bins that are sorted.  A bin that does not fit the registers all the same is
+// sorted by its workgroup through global memory (bucket_sort_long): slow, and correct.
+// Elements travel as they came in (the key is derived where it is needed), so a stable sort
+// keeps the bit patterns of zeros and NaNs in input order with no patching afterwards; complex
+// keys, which are not cheap to derive, travel as keys with the elements as their payload.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "lanes.hpp"
+
+namespace misort {
+
+constexpr int BK_SLOTS      = 256;  // splitter table: 255 splitters at most, padded with the largest key
+constexpr int BK_BINS       = 512;
+constexpr int BK_OVERSAMPLE = 16;   // samples per splitter interval
+constexpr int BK_PLAN_NT    = 1024;  // the planning workgroup sorts up to 1024 * 4 sample keys
+constexpr int BK_PLAN_IPT   = 4;
+constexpr int BK_COUNT_NT   = 1024;
+constexpr int BK_NT         = 1024;  // scatter and bin sort
+
+struct BucketParams {
+  const void* keys_in;   // the row, elements as they came in
+  const void* pay_in;    // PAY_I64: the caller's payload; else unused (positions are made up)
+  void* keys_out;        // sorted elements, or NULL
+  void* pay_out;         // int64 payload / positions (+ index_offset), or NULL
+  void* buf_keys[2];     // scratch: the row in bin order ([1]: second buffer for long bins)
+  void* buf_pay[2];      // scratch: its payload (u32 positions or int64)
+  void* splitters;       // KeyT[BK_SLOTS], ascending keys, written by the plan kernel
+  uint32_t* chunk_hist;  // [n_chunks][BK_BINS]
+  uint32_t* slab_tot;    // [n_slabs][BK_BINS], cleared by the plan kernel
+  uint32_t* bin_start;   // [BK_BINS + 1] first position of every bin, written by chunk 0 of the scatter
+  uint32_t n;            // elements in the row
+  uint32_t n_split;      // splitters in use
+  uint32_t tile, tiles_per_chunk, n_chunks, chunks_per_slab, n_slabs;
+  uint32_t cap;          // longest bin sorted in registers
+  int64_t index_offset;
+  int xform;             // of the elements in keys_in
+  int keys_travel;       // 1: the scatter writes keys (complex), 0: the elements themselves
+  int rank_by_add;
+  int dbg_max_bits;
+  int direct_equal;      // 1: the scatter writes the bins of equal keys straight to the outputs
+                         // (outputs do not alias the inputs); 0: the bin sort copies them
+};
+
+// Rank of this lane's key among the keys with the same digit value that the wavefront has
+// ranked so far (earlier calls, lower lanes of this one); my_hist: the wavefront's counters in
+// LDS.  by_add: one returning add, which relies on the LDS serving the lanes of one instruction
+// that hit the same word in ascending lane order (the library checks that once per GPU);
+// otherwise the lanes with the same value find each other with one ballot per digit bit.
+// Every lane of the wavefront must be active; lanes with valid == false hold no key.
+template <int BITS>
+__device__ __forceinline__ uint32_t wave_rank(uint32_t* my_hist, uint32_t d, bool valid, int by_add)
+{
+  if (by_add) return valid ? atomicAdd(&my_hist[d], 1u) : 0u;
+  uint64_t peers = __ballot(valid);
+#pragma unroll
+  for (int b = 0; b < BITS; ++b) {
+    const bool bit    = (d >> b) & 1u;
+    const uint64_t bl = __ballot(bit);
+    peers &= bit ? bl : ~bl;
+  }
+  const uint32_t below =
+    __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+  const uint32_t cnt = (uint32_t)__popcll(peers);
+  // the lowest peer adds the group's size; LDS runs a wavefront's operations in order, so the
+  // read that follows sees the counter after this call and no later one
+  if (valid && below == 0) atomicAdd(&my_hist[d], cnt);
+  const uint32_t after = __hip_atomic_load(&my_hist[d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return after - cnt + below;
+}
+
+// ---------------------------------------------------------------------------------------
+// splitter table in LDS: the sorted splitters and the same keys laid out as a search tree
+// ---------------------------------------------------------------------------------------
+template <typename KeyT>
+struct SplitterTable {
+  KeyT sorted[BK_SLOTS];  // [j] = splitter j; unused slots and [255] hold the largest key
+  KeyT tree[BK_SLOTS];    // node j (1 .. 255) of a complete binary tree over sorted[0 .. 254]
+};
+
+template <typename KeyT, int NT>
+__device__ __forceinline__ void load_splitters(SplitterTable<KeyT>& t, const KeyT* spl)
+{
+  for (int j = threadIdx.x; j < BK_SLOTS; j += NT) t.sorted[j] = spl[j];
+  __syncthreads();
+  for (int j = threadIdx.x; j < BK_SLOTS; j += NT) {
+    if (j == 0) {
+      t.tree[0] = t.sorted[0];  // never read
+    } else {
+      const int l   = 31 - __builtin_clz((unsigned)j);
+      const int pos = j - (1 << l);
+      t.tree[j]     = t.sorted[((2 * pos + 1) << (7 - l)) - 1];
+    }
+  }
+  __syncthreads();
+}
+
+// Bin of a key: twice the number of splitters below it, plus one if it equals the next one.
+template <typename KeyT>
+__device__ __forceinline__ uint32_t bin_of(const SplitterTable<KeyT>& t, KeyT k)
+{
+  uint32_t j = 1;
+#pragma unroll
+  for (int l = 0; l < 8; ++l) j = 2 * j + (k > t.tree[j] ? 1u : 0u);
+  j -= BK_SLOTS;
+  return 2 * j + (t.sorted[j] == k ? 1u : 0u);
+}
+
+// ---------------------------------------------------------------------------------------
+// radix sort of up to NT * IPT elements held by a workgroup, least significant digit first.
+// The len elements lie in rows of 64; every wavefront owns R consecutive rows, R just large
+// enough that the NT / 64 wavefronts cover them all (a short bin is spread over all wavefronts:
+// a wavefront alone on its SIMD issues an instruction only every dozen clocks).  Element
+// e = (wave * R + i) * 64 + lane sits in slot i < R of its thread.  Sorts by the bits
+// [0, nbits) of to_key(element, xform) - base.
+// ---------------------------------------------------------------------------------------
+template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT>
+struct BlockSortSmem {
+  uint32_t whist[(NT / 64) * RADIX];
+  uint32_t wave_tot[NT / 64];
+  __attribute__((aligned(16))) KeyT keys[NT * IPT];
+  __attribute__((aligned(16))) PayT pay[HAS_PAY ? NT * IPT : 1];
+};
+
+struct BlockSortGeom {
+  uint32_t rows;   // rows of 64 elements in use
+  uint32_t R;      // rows per wavefront
+  uint32_t wbase;  // element of this thread's slot 0
+};
+template <int NT>
+__device__ __forceinline__ BlockSortGeom block_sort_geom(uint32_t len)
+{
+  BlockSortGeom g;
+  g.rows  = (len + 63) / 64;
+  g.R     = (g.rows + NT / 64 - 1) / (NT / 64);
+  g.wbase = (threadIdx.x >> 6) * g.R * 64 + (threadIdx.x & 63);
+  return g;
+}
+
+template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT>
+__device__ __forceinline__ void block_radix_sort(uint32_t* whist /* (NT / 64) * RADIX */,
+                                                 uint32_t* wave_tot /* NT / 64 */,
+                                                 KeyT* skeys /* NT * IPT */, PayT* spay /* NT * IPT */,
+                                                 KeyT (&el)[IPT], PayT (&pay)[HAS_PAY ? IPT : 1],
+                                                 uint32_t len, KeyT base, int nbits, int xform, int by_add)
+{
+  static_assert(NT % RADIX == 0, "whole groups of one thread per digit value");
+  constexpr int NW  = NT / 64;
+  constexpr int NG  = NT / RADIX;  // thread groups, each covering all digit values
+  constexpr int WPG = NW / NG;     // wavefronts whose counters a group rewrites
+  const int tid          = threadIdx.x;
+  const int lane         = tid & 63;
+  const int wave         = tid >> 6;
+  const BlockSortGeom g  = block_sort_geom<NT>(len);
+  const uint32_t R       = g.R;
+  const uint32_t wbase   = g.wbase;
+  uint32_t* my_hist      = whist + wave * RADIX;
+  const uint32_t dv      = tid & (RADIX - 1);
+  const int grp          = wave / (RADIX / 64);
+  for (int shift = 0; shift < nbits; shift += RADIX_BITS) {
+    for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
+    __syncthreads();
+    uint32_t d[IPT], r[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      if ((uint32_t)i < R && (uint32_t)wave * R + i < g.rows) {
+        const bool valid = wbase + i * 64 < len;
+        const KeyT k     = valid ? (KeyT)(KeyOps<KeyT>::to_key(el[i], xform) - base) : KeyOps<KeyT>::max_key();
+        d[i]             = KeyOps<KeyT>::digit(k, shift);
+        r[i]             = wave_rank<RADIX_BITS>(my_hist, d[i], valid, by_add);
+      }
+    }
+    __syncthreads();
+    // every thread takes digit value dv and the wavefronts of its group; all groups add up the
+    // value's count over every wavefront and scan the counts over the digit values for themselves
+    uint32_t count = 0, before = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      if (w == grp * WPG) before = count;
+      count += whist[w * RADIX + dv];
+    }
+    const uint32_t incl = wave_incl_scan_u32(count);
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    {
+      uint32_t off = incl - count + before;
+      for (int w = grp * (RADIX / 64); w < wave; ++w) off += wave_tot[w];
+      uint32_t* mine = whist + grp * WPG * RADIX + dv;
+#pragma unroll
+      for (int w = 0; w < WPG; ++w) {
+        const uint32_t c = mine[w * RADIX];
+        mine[w * RADIX]  = off;
+        off += c;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      if ((uint32_t)i < R && wbase + i * 64 < len) {
+        const uint32_t q = my_hist[d[i]] + r[i];
+        skeys[q]         = el[i];
+        if constexpr (HAS_PAY) spay[q] = pay[i];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      if ((uint32_t)i < R && wbase + i * 64 < len) {
+        el[i] = skeys[wbase + i * 64];
+        if constexpr (HAS_PAY) pay[i] = spay[wbase + i * 64];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// plan: splitters from a sorted sample; also clears the slab totals of the count kernel
+// ---------------------------------------------------------------------------------------
+template <typename KeyT>
+__global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
+{
+  constexpr int NT = BK_PLAN_NT, IPT = BK_PLAN_IPT;
+  __shared__ BlockSortSmem<KeyT, uint32_t, false, NT, IPT> sm;
+  const int tid = threadIdx.x;
+  for (uint32_t i = tid; i < p.n_slabs * BK_BINS; i += NT) p.slab_tot[i] = 0;
+  // sample e of S comes from its own stretch of n / S elements, at a place inside it that a hash
+  // of e picks (evenly spaced places would meet periodic data at the same phase every time)
+  const uint32_t S     = (p.n_split + 1) * BK_OVERSAMPLE;  // <= NT * IPT
+  const uint32_t span  = p.n / S > 0 ? p.n / S : 1;
+  const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
+  const BlockSortGeom g = block_sort_geom<NT>(S);
+  KeyT k[IPT];
+  uint32_t nopay[1];
+#pragma unroll
+  for (int i = 0; i < IPT; ++i) {
+    const uint32_t e = g.wbase + i * 64;
+    uint32_t h       = e * 0x9E3779B1u;
+    h ^= h >> 15;
+    h *= 0x85EBCA77u;
+    h ^= h >> 13;
+    uint64_t pos = (uint64_t)e * p.n / S + h % span;
+    if (pos >= p.n) pos = p.n - 1;
+    k[i] = ((uint32_t)i < g.R && e < S) ? KeyOps<KeyT>::to_key(in[pos], p.xform) : KeyOps<KeyT>::max_key();
+  }
+  block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
+                                                   (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add);
+  // the sorted sample is still in sm.keys; splitter t = sample 16 (t + 1) - 1
+  KeyT* spl = reinterpret_cast<KeyT*>(p.splitters);
+  for (uint32_t t = tid; t < BK_SLOTS; t += NT)
+    spl[t] = t < p.n_split ? sm.keys[(t + 1) * BK_OVERSAMPLE - 1] : KeyOps<KeyT>::max_key();
+}
+
+// ---------------------------------------------------------------------------------------
+// count: keys per bin of every chunk, added up per slab of chunks
+// ---------------------------------------------------------------------------------------
+template <typename KeyT>
+__global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams p)
+{
+  constexpr int NT = BK_COUNT_NT, NW = NT / 64;
+  __shared__ SplitterTable<KeyT> tab;
+  __shared__ uint32_t hist[NW * BK_BINS];
+  const int tid = threadIdx.x, wave = tid >> 6;
+  for (int i = tid; i < NW * BK_BINS; i += NT) hist[i] = 0;
+  load_splitters<KeyT, NT>(tab, reinterpret_cast<const KeyT*>(p.splitters));
+  const uint32_t chunk = blockIdx.x;
+  const uint64_t clen  = (uint64_t)p.tiles_per_chunk * p.tile;
+  const uint64_t b0    = (uint64_t)chunk * clen;
+  const uint64_t b1    = b0 + clen < p.n ? b0 + clen : p.n;
+  const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
+  uint32_t* my         = hist + wave * BK_BINS;
+  // (four independent loads, then four searches side by side)
+  for (uint64_t i0 = b0; i0 < b1; i0 += 4 * NT) {
+    KeyT raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint64_t i = i0 + (uint64_t)u * NT + tid;
+      raw[u]           = in[i < b1 ? i : b0];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint64_t i = i0 + (uint64_t)u * NT + tid;
+      const uint32_t b = bin_of(tab, KeyOps<KeyT>::to_key(raw[u], p.xform));
+      if (i < b1) atomicAdd(&my[b], 1u);
+    }
+  }
+  __syncthreads();
+  uint32_t* out  = p.chunk_hist + (uint64_t)chunk * BK_BINS;
+  uint32_t* slab = p.slab_tot + (uint64_t)(chunk / p.chunks_per_slab) * BK_BINS;
+  for (int b = tid; b < BK_BINS; b += NT) {
+    uint32_t c = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) c += hist[w * BK_BINS + b];
+    out[b] = c;
+    if (c) atomicAdd(&slab[b], c);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// scatter: the elements of every chunk to their bins, in input order
+// ---------------------------------------------------------------------------------------
+template <typename KeyT, int PAY, int IPT>
+__global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
+{
+  constexpr int NT = BK_NT, NW = NT / 64, TILE = NT * IPT;
+  using PayT = typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type;
+  constexpr bool HAS_PAY = PAY != PAY_NONE;
+  static_assert(TILE <= 65535, "the staged bin of an element is a 16-bit word");
+  __shared__ SplitterTable<KeyT> tab;
+  __shared__ uint32_t whist[NW * BK_BINS];
+  __shared__ uint32_t bin_base[BK_BINS];  // first staged slot of every bin in the tile
+  __shared__ uint32_t gpos[BK_BINS];      // where the chunk's next element of every bin goes
+  __shared__ uint32_t wave_tot[BK_BINS / 64];
+  __shared__ __attribute__((aligned(16))) KeyT skeys[TILE];
+  __shared__ __attribute__((aligned(16))) PayT spay[HAS_PAY ? TILE : 1];
+  __shared__ uint16_t sbin[TILE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t wbase = (uint32_t)wave * (64 * IPT) + lane;
+  const uint32_t chunk = blockIdx.x;
+  load_splitters<KeyT, NT>(tab, reinterpret_cast<const KeyT*>(p.splitters));
+
+  // ---- where this chunk's elements of every bin start: the bins before (all chunks), the
+  // same bin in the slabs before this chunk's and in the chunks before it inside its slab
+  {
+    uint32_t tot = 0, before = 0;
+    if (tid < BK_BINS) {
+      const uint32_t slab = chunk / p.chunks_per_slab;
+      for (uint32_t s = 0; s < p.n_slabs; ++s) {
+        const uint32_t v = p.slab_tot[(uint64_t)s * BK_BINS + tid];
+        tot += v;
+        if (s < slab) before += v;
+      }
+      for (uint32_t c = slab * p.chunks_per_slab; c < chunk; ++c) before += p.chunk_hist[(uint64_t)c * BK_BINS + tid];
+    }
+    const uint32_t incl = wave_incl_scan_u32(tot);
+    if (tid < BK_BINS && lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    if (tid < BK_BINS) {
+      uint32_t start = incl - tot;
+      for (int w = 0; w < wave; ++w) start += wave_tot[w];
+      gpos[tid] = start + before;
+      if (chunk == 0) {
+        p.bin_start[tid] = start;
+        if (tid == BK_BINS - 1) p.bin_start[BK_BINS] = p.n;
+      }
+    }
+    __syncthreads();
+  }
+
+  const KeyT* in   = reinterpret_cast<const KeyT*>(p.keys_in);
+  KeyT* kbuf       = reinterpret_cast<KeyT*>(p.buf_keys[0]);
+  PayT* pbuf       = reinterpret_cast<PayT*>(p.buf_pay[0]);
+  KeyT* kout       = reinterpret_cast<KeyT*>(p.keys_out);
+  int64_t* pout    = reinterpret_cast<int64_t*>(p.pay_out);
+  uint32_t* my_hist = whist + wave * BK_BINS;
+  const uint32_t tile0 = chunk * p.tiles_per_chunk;
+  const uint32_t tiles = (p.n + TILE - 1) / TILE;
+  uint32_t tile_end    = tile0 + p.tiles_per_chunk;
+  if (tile_end > tiles) tile_end = tiles;
+
+  for (uint32_t t = tile0; t < tile_end; ++t) {
+    const uint32_t t0    = t * TILE;
+    const uint32_t valid = p.n - t0 < (uint32_t)TILE ? p.n - t0 : (uint32_t)TILE;
+    KeyT el[IPT];
+    PayT pv[HAS_PAY ? IPT : 1];
+    uint32_t b[IPT], r[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e = wbase + i * 64;
+      el[i]            = in[t0 + (e < valid ? e : 0u)];
+      if constexpr (PAY == PAY_I64) pv[i] = reinterpret_cast<const int64_t*>(p.pay_in)[t0 + (e < valid ? e : 0u)];
+      if constexpr (PAY == PAY_IDX32) pv[i] = t0 + e;
+    }
+    for (int i = tid; i < NW * BK_BINS; i += NT) whist[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e = wbase + i * 64;
+      const KeyT k     = KeyOps<KeyT>::to_key(el[i], p.xform);
+      if (p.keys_travel) el[i] = k;
+      // (slots past the end of the row in the last tile hold no key)
+      b[i] = e < valid ? bin_of(tab, k) : (uint32_t)(BK_BINS - 1);
+      r[i] = wave_rank<9>(my_hist, b[i], e < valid, p.rank_by_add);
+    }
+    __syncthreads();
+    uint32_t tot = 0;
+    if (tid < BK_BINS) {
+#pragma unroll
+      for (int w = 0; w < NW; ++w) tot += whist[w * BK_BINS + tid];
+    }
+    const uint32_t incl = wave_incl_scan_u32(tot);
+    if (tid < BK_BINS && lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    if (tid < BK_BINS) {
+      uint32_t run = incl - tot;
+      for (int w = 0; w < wave; ++w) run += wave_tot[w];
+      bin_base[tid] = run;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const uint32_t c            = whist[w * BK_BINS + tid];
+        whist[w * BK_BINS + tid] = run;
+        run += c;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      if (wbase + i * 64 < valid) {
+        const uint32_t q = my_hist[b[i]] + r[i];
+        skeys[q]         = el[i];
+        if constexpr (HAS_PAY) spay[q] = pv[i];
+        sbin[q] = (uint16_t)b[i];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t q = (uint32_t)tid + i * NT;
+      if (q < valid) {
+        const uint32_t bin = sbin[q];
+        const uint32_t dst = gpos[bin] + (q - bin_base[bin]);
+        if (p.direct_equal && (bin & 1u)) {
+          if (kout) kout[dst] = skeys[q];  // (keys_out is NULL where keys travel)
+          if constexpr (PAY == PAY_IDX32) pout[dst] = (int64_t)spay[q] + p.index_offset;
+          if constexpr (PAY == PAY_I64) pout[dst] = spay[q];
+        } else {
+          kbuf[dst] = skeys[q];
+          if constexpr (HAS_PAY) pbuf[dst] = spay[q];
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < BK_BINS) gpos[tid] += tot;
+    // (the next tile's first barrier comes before anything reads gpos again)
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// bin sort
+// ---------------------------------------------------------------------------------------
+// A bin too long for the registers: plain LSD passes by this one workgroup between the two
+// scratch buffers, NT elements at a time.  Splitters from a sorted sample leave this to inputs
+// built against the sampling; it is here so that those are sorted too.
+template <typename KeyT, int PAY>
+__device__ void bucket_sort_long(const BucketParams& p, uint32_t start, uint32_t len, KeyT base, int nbits,
+                                 int xform, uint32_t* whist /* (NT / 64) * RADIX */,
+                                 uint32_t* gbase /* RADIX */, uint32_t* wave_tot /* RADIX / 64 */)
+{
+  constexpr int NT = BK_NT, NW = NT / 64;
+  using PayT = typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t* my_hist = whist + wave * RADIX;
+  KeyT* kout        = reinterpret_cast<KeyT*>(p.keys_out);
+  int64_t* pout     = reinterpret_cast<int64_t*>(p.pay_out);
+  int cur           = 0;
+  for (int shift = 0; shift < nbits; shift += RADIX_BITS) {
+    const bool last  = shift + RADIX_BITS >= nbits;
+    const KeyT* ksrc = reinterpret_cast<const KeyT*>(p.buf_keys[cur]) + start;
+    const PayT* psrc = reinterpret_cast<const PayT*>(p.buf_pay[cur]) + start;
+    KeyT* kdst       = reinterpret_cast<KeyT*>(p.buf_keys[cur ^ 1]) + start;
+    PayT* pdst       = reinterpret_cast<PayT*>(p.buf_pay[cur ^ 1]) + start;
+    // counts of this digit over the bin, then where every digit value starts
+    for (int i = tid; i < RADIX; i += NT) gbase[i] = 0;
+    __syncthreads();
+    for (uint32_t e = tid; e < len; e += NT)
+      atomicAdd(&gbase[KeyOps<KeyT>::digit((KeyT)(KeyOps<KeyT>::to_key(ksrc[e], xform) - base), shift)], 1u);
+    __syncthreads();
+    {
+      const uint32_t c    = tid < RADIX ? gbase[tid] : 0u;
+      const uint32_t incl = wave_incl_scan_u32(c);
+      if (tid < RADIX && lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      if (tid < RADIX) {
+        uint32_t s = incl - c;
+        for (int w = 0; w < wave; ++w) s += wave_tot[w];
+        gbase[tid] = s;
+      }
+      __syncthreads();
+    }
+    for (uint32_t t0 = 0; t0 < len; t0 += NT) {
+      const uint32_t e = t0 + tid;
+      const bool valid = e < len;
+      const KeyT el    = ksrc[valid ? e : 0u];
+      PayT pv{};
+      if constexpr (PAY != PAY_NONE) pv = psrc[valid ? e : 0u];
+      const uint32_t d = valid ? KeyOps<KeyT>::digit((KeyT)(KeyOps<KeyT>::to_key(el, xform) - base), shift) : 0u;
+      for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
+      __syncthreads();
+      const uint32_t r = wave_rank<RADIX_BITS>(my_hist, d, valid, p.rank_by_add);
+      __syncthreads();
+      uint32_t tot = 0;
+      if (tid < RADIX) {
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+          const uint32_t c       = whist[w * RADIX + tid];
+          whist[w * RADIX + tid] = tot;
+          tot += c;
+        }
+      }
+      __syncthreads();
+      if (valid) {
+        const uint32_t dst = gbase[d] + my_hist[d] + r;
+        if (last) {
+          if (kout) kout[start + dst] = el;
+          if constexpr (PAY == PAY_IDX32) pout[start + dst] = (int64_t)pv + p.index_offset;
+          if constexpr (PAY == PAY_I64) pout[start + dst] = pv;
+        } else {
+          kdst[dst] = el;
+          if constexpr (PAY != PAY_NONE) pdst[dst] = pv;
+        }
+      }
+      __syncthreads();
+      if (tid < RADIX) gbase[tid] += tot;
+      __syncthreads();
+    }
+    // what this pass wrote to global memory is read by other threads of the workgroup next
+    __threadfence();
+    __syncthreads();
+    cur ^= 1;
+  }
+}
+
+// grid: one workgroup per pair of bins (2g: the keys between two splitters, sorted here;
+// 2g + 1: the keys equal to splitter g, which only need copying, and only if the scatter
+// could not write them to the outputs itself).
+template <typename KeyT, int PAY, int IPT>
+__global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
+{
+  constexpr int NT = BK_NT, CAP = NT * IPT;
+  using PayT = typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type;
+  constexpr bool HAS_PAY = PAY != PAY_NONE;
+  __shared__ BlockSortSmem<KeyT, PayT, HAS_PAY, NT, IPT> sm;
+  __shared__ uint32_t gbase[RADIX];
+  const int tid = threadIdx.x;
+  const uint32_t g     = blockIdx.x;
+  const uint32_t start = p.bin_start[2 * g], mid = p.bin_start[2 * g + 1], end = p.bin_start[2 * g + 2];
+  const uint32_t len   = mid - start;
+  const KeyT* kbuf     = reinterpret_cast<const KeyT*>(p.buf_keys[0]);
+  const PayT* pbuf     = reinterpret_cast<const PayT*>(p.buf_pay[0]);
+  KeyT* kout           = reinterpret_cast<KeyT*>(p.keys_out);
+  int64_t* pout        = reinterpret_cast<int64_t*>(p.pay_out);
+  auto emit = [&](uint32_t dst, KeyT el, PayT pv) {
+    if (kout) kout[dst] = el;
+    if constexpr (PAY == PAY_IDX32) pout[dst] = (int64_t)pv + p.index_offset;
+    if constexpr (PAY == PAY_I64) pout[dst] = pv;
+  };
+  if (!p.direct_equal) {
+    for (uint32_t e = mid + tid; e < end; e += NT) emit(e, kbuf[e], HAS_PAY ? pbuf[HAS_PAY ? e : 0] : PayT{});
+  }
+  if (len == 0) return;
+  // the keys of the bin lie strictly between the splitters lo and hi: sorted by key - lo, which
+  // is below hi - lo and so has that many bits at most
+  const KeyT* spl = reinterpret_cast<const KeyT*>(p.splitters);
+  const KeyT lo   = g > 0 ? spl[g - 1] : (KeyT)0;
+  const KeyT hi   = spl[g];
+  const unsigned long long diff = (unsigned long long)(KeyT)(hi - lo);
+  int nbits = diff ? 64 - __builtin_clzll(diff) : 0;
+  if (p.dbg_max_bits >= 0 && nbits > p.dbg_max_bits) nbits = p.dbg_max_bits;
+  const int xform = p.keys_travel ? (int)XF_UNSIGNED : p.xform;
+  if (len > p.cap) {
+    bucket_sort_long<KeyT, PAY>(p, start, len, lo, nbits > 0 ? nbits : 1, xform, sm.whist, gbase, sm.wave_tot);
+    return;
+  }
+  const BlockSortGeom geo = block_sort_geom<NT>(len);
+  KeyT el[IPT];
+  PayT pv[HAS_PAY ? IPT : 1];
+#pragma unroll
+  for (int i = 0; i < IPT; ++i) {
+    const uint32_t e = geo.wbase + i * 64;
+    if ((uint32_t)i < geo.R && e < len) {
+      el[i] = kbuf[start + e];
+      if constexpr (HAS_PAY) pv[i] = pbuf[start + e];
+    }
+  }
+  block_radix_sort<KeyT, PayT, HAS_PAY, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, el, pv, len, lo, nbits,
+                                                 xform, p.rank_by_add);
+#pragma unroll
+  for (int i = 0; i < IPT; ++i) {
+    const uint32_t e = geo.wbase + i * 64;
+    if ((uint32_t)i < geo.R && e < len) emit(start + e, el[i], HAS_PAY ? pv[HAS_PAY ? i : 0] : PayT{});
+  }
+}
+
+}  // namespace misort

@@ -4,9 +4,11 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <mutex>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <string>
 #include <type_traits>
 #include <vector>
@@ -22,6 +24,7 @@
 #include "select.hpp"
 #include "unique.hpp"
 #include "selftest.hpp"
+#include "bucket.hpp"
 
 namespace misort {
 
@@ -29,15 +32,68 @@ static_assert(PAY_I64 == 2, "rows_api.hpp spells the caller-payload kind as 2");
 
 thread_local std::string g_last_error;
 
-// Ranking by returning LDS adds (radix.hpp, rank_by_add) is on unless the environment says
-// MISORT_RANK_BALLOT=1 when the library is first used; read once, never changed afterwards.
-static int rank_by_add_default()
+static constexpr int kMaxDevices = 64;
+
+// Ranking by returning LDS adds (radix.hpp, rank_by_add) leans on the LDS serving the lanes of
+// one instruction that hit the same word in ascending lane order, which gfx950 does and no
+// manual promises.  So the library decides per GPU, the first time a sort runs there (or in
+// misort_init): ballots if the environment says MISORT_RANK_BALLOT=1 (read once), ballots on
+// anything that is not gfx950, and otherwise a short probe on a stream of its own (three
+// launches of lds_lane_order_probe_kernel, 25 million lane operations with 256, 4 and 1
+// distinct words per wavefront, about 0.1 ms) that compares the returning add with the ballot
+// match lane by lane: adds only if not one lane disagrees.  The verdict is kept per GPU.
+enum RankMode : int { RANK_UNTESTED = 0, RANK_ADD = 1, RANK_BALLOT = 2 };
+static std::atomic<int> g_rank_mode[kMaxDevices];
+static std::mutex g_probe_mutex;  // the probe's counters are one pair per GPU
+
+static bool rank_ballot_env()
 {
-  static const int v = [] {
+  static const bool v = [] {
     const char* e = getenv("MISORT_RANK_BALLOT");
-    return (e && *e && *e != '0') ? 0 : 1;
+    return e && *e && *e != '0';
   }();
   return v;
+}
+
+static int probe_lane_order(int dev)
+{
+  std::lock_guard<std::mutex> lock(g_probe_mutex);
+  int m = g_rank_mode[dev].load(std::memory_order_acquire);
+  if (m != RANK_UNTESTED) return m;
+  m = RANK_BALLOT;  // whatever goes wrong below: ballots need no such property
+  hipDeviceProp_t prop;
+  hipStream_t st = nullptr;
+  unsigned long long* counts = nullptr;
+  if (hipGetDeviceProperties(&prop, dev) == hipSuccess && strncmp(prop.gcnArchName, "gfx950", 6) == 0 &&
+      hipGetSymbolAddress(reinterpret_cast<void**>(&counts), HIP_SYMBOL(g_selftest_counts)) == hipSuccess &&
+      hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess) {
+    hipLaunchKernelGGL(store_u64_kernel, dim3(1), dim3(1), 0, st, counts, 0ull);
+    hipLaunchKernelGGL(store_u64_kernel, dim3(1), dim3(1), 0, st, counts + 1, 0ull);
+    const uint32_t masks[3] = {0xFFu, 0x03u, 0x00u};
+    for (int i = 0; i < 3; ++i)
+      hipLaunchKernelGGL(lds_lane_order_probe_kernel, dim3(256), dim3(1024), 0, st, 32u, masks[i],
+                         0x2468ACEu + i, counts);
+    unsigned long long h[2] = {0, 1};
+    hipError_t e = hipMemcpyAsync(h, counts, sizeof h, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e == hipSuccess && hipGetLastError() == hipSuccess && h[0] == 3ull * 256 * 16 * 32 * 64 && h[1] == 0)
+      m = RANK_ADD;
+  }
+  if (st) hipStreamDestroy(st);
+  (void)hipGetLastError();
+  g_rank_mode[dev].store(m, std::memory_order_release);
+  return m;
+}
+
+// 1: this GPU ranks with returning adds, 0: with ballots
+static int rank_by_add_on_current_device()
+{
+  if (rank_ballot_env()) return 0;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int m = g_rank_mode[dev].load(std::memory_order_acquire);
+  if (m == RANK_UNTESTED) m = probe_lane_order(dev);
+  return m == RANK_ADD ? 1 : 0;
 }
 
 // The digit side-band of keys-only sorts (radix.hpp, SIDE) is on unless the environment says
@@ -63,14 +119,26 @@ static bool skip_passes_default()
 }
 
 // From how many bytes of keys on the last pass whose digit varies writes the result (it costs
-// one more launch per middle pass).  MISORT_EARLY_LAST_BYTES in the environment overrides the
-// 256 MB; read at every call, so that tests can reach the path with small arrays.
-static size_t early_last_min_bytes()
+// one more launch per middle pass): 256 MB, or what MISORT_EARLY_LAST_BYTES said when the
+// library was first used, or what the caller of a *_opts entry point says for that call.
+static size_t early_last_min_bytes_default()
 {
-  const char* e = getenv("MISORT_EARLY_LAST_BYTES");
-  if (e && *e) return (size_t)strtoull(e, nullptr, 10);
-  return (size_t)1 << 28;
+  static const size_t v = [] {
+    const char* e = getenv("MISORT_EARLY_LAST_BYTES");
+    return (e && *e) ? (size_t)strtoull(e, nullptr, 10) : (size_t)1 << 28;
+  }();
+  return v;
 }
+
+// What the *_opts entry points let a caller choose per call (misort_options in misort.h);
+// everything else runs with the defaults.
+struct PlanOptions {
+  size_t target_chunks = 0;             // 0: the built-in choice
+  long long early_last_min_bytes = -1;  // < 0: the default above
+  int bucket_path = -1;                 // < 0: the built-in choice; 0: never; > 0: wherever it is able to run
+  unsigned bucket_bins = 0;             // 0: the built-in choice; else splitter intervals, 2 .. 256
+  unsigned bucket_cap = 0;              // 0: the built-in choice; else the longest bin sorted in registers
+};
 
 static int fail(int code, const std::string& msg)
 {
@@ -110,6 +178,10 @@ enum KernelId : int {
   K_SELECT_EMIT,
   K_SPLIT,
   K_COLSORT,
+  K_BUCKET_PLAN,
+  K_BUCKET_COUNT,
+  K_BUCKET_SCATTER,
+  K_BUCKET_SORT,
   K_NUM
 };
 
@@ -122,7 +194,8 @@ static const char* const kKernelNames[K_NUM] = {
   "unique_count",    "unique_offsets",  "unique_compact",   "count8_hist",
   "count8_fill",     "select_init",     "select_hist",      "select_pick",
   "select_counts",   "select_above",    "select_emit",    "select_split",
-  "colsort_wave"};
+  "colsort_wave",    "bucket_plan",     "bucket_count",     "bucket_scatter",
+  "bucket_sort"};
 
 // ---------------------------------------------------------------------------------------
 // dtype table
@@ -156,17 +229,13 @@ static bool dtype_info(int dtype, DtypeInfo& d)
 // ---------------------------------------------------------------------------------------
 // plan
 // ---------------------------------------------------------------------------------------
-enum Strategy : int { S_EMPTY = 0, S_ROW_WAVE, S_ROW_BLOCK, S_RADIX, S_COUNT16, S_COUNT8 };
+enum Strategy : int { S_EMPTY = 0, S_ROW_WAVE, S_ROW_BLOCK, S_RADIX, S_COUNT16, S_COUNT8, S_BUCKET };
 
 // Tile shape of the downsweep per key width and payload kind: threads, keys per thread,
 // elements per 128-byte output line kept in the carry (G), workgroups per CU.  One
 // workgroup of 1024 threads fills a CU: staging + carry take most of its 160 KB of LDS.
-#ifndef MISORT_NT
-#define MISORT_NT 1024
-#endif
-#ifndef MISORT_OCC
-#define MISORT_OCC 1
-#endif
+constexpr int kTileThreads = 1024;
+constexpr int kTileOcc     = 1;
 constexpr int pay_bytes_of(int pay) { return pay == PAY_NONE ? 0 : (pay == PAY_IDX32 ? 4 : 8); }
 constexpr int carry_group(int kb, int pay)
 {
@@ -176,40 +245,28 @@ constexpr int carry_group(int kb, int pay)
   const int narrow  = (pb != 0 && pb < kb) ? pb : kb;
   int g             = 128 / narrow;
   while (256 * g * (kb + pb) > 64 * 1024) g /= 2;
-#ifdef MISORT_G
-  if (g > MISORT_G) g = MISORT_G;
-#endif
   return g;
 }
 constexpr int items_per_thread(int kb, int pay, int nt)
 {
   // staging + carry + per-wave counters + bookkeeping within 160 KB
   const int pb     = pay_bytes_of(pay);
-  const int budget = 160 * 1024 / MISORT_OCC - 256 * carry_group(kb, pay) * (kb + pb) -
+  const int budget = 160 * 1024 / kTileOcc - 256 * carry_group(kb, pay) * (kb + pb) -
                      (nt / 64) * 1024 - 6 * 1024;
   int ipt          = budget / (nt * (kb + pb));
   // two key buffers (current and next tile) + payload + ranks stay in registers
-#ifndef MISORT_IPT_KEYS
-#define MISORT_IPT_KEYS 16
-#endif
-#ifndef MISORT_IPT_IDX
-#define MISORT_IPT_IDX 8
-#endif
-#ifndef MISORT_IPT_KEYS8
-#define MISORT_IPT_KEYS8 8
-#endif
-  const int cap = kb <= 4 ? (pb == 8 ? 6 : (pb == 0 ? MISORT_IPT_KEYS : MISORT_IPT_IDX))
-                          : (kb == 8 ? (pb == 8 ? 4 : (pb == 0 ? MISORT_IPT_KEYS8 : 7)) : (pb == 8 ? 3 : 4));
+  const int cap = kb <= 4 ? (pb == 8 ? 6 : (pb == 0 ? 16 : 8))
+                          : (kb == 8 ? (pb == 8 ? 4 : (pb == 0 ? 8 : 7)) : (pb == 8 ? 3 : 4));
   if (ipt > cap) ipt = cap;
   if (ipt < 1) ipt = 1;
   return ipt;
 }
 template <int KEYBYTES, int PAY>
 struct TileCfg {
-  static constexpr int NT  = MISORT_NT;
+  static constexpr int NT  = kTileThreads;
   static constexpr int G   = carry_group(KEYBYTES, PAY);
   static constexpr int IPT = items_per_thread(KEYBYTES, PAY, NT);
-  static constexpr int OCC = MISORT_OCC;
+  static constexpr int OCC = kTileOcc;
   static_assert(IPT >= 1, "tile does not fit");
 };
 
@@ -272,29 +329,25 @@ struct Plan {
   size_t off_gather_idx = 0, off_gather_src = 0;
   // counting sort of 2-byte keys: chunks of the histogram kernel, counters, their scan
   size_t c16_chunks = 0, c16_chunk_len = 0, off_c16_hist = 0, off_c16_prefix = 0;
+  // sample -> count -> scatter -> sort the bins (bucket.hpp): geometry and scratch
+  uint32_t bk_split = 0, bk_cap = 0, bk_tile = 0, bk_tiles_per_chunk = 0, bk_chunks = 0, bk_slabs = 0;
+  size_t off_bk_splitters = 0, off_bk_slab_tot = 0, off_bk_chunk_hist = 0, off_bk_bin_start = 0;
   size_t total = 0;
 };
+
+// Slots per thread of the bin sort (1024 threads): the bin and its payload are staged in LDS
+// between the passes, 128 KB of it.
+constexpr int bucket_sort_ipt(int kb, int pay) { return kb + pay_bytes_of(pay) <= 8 ? 16 : 8; }
+constexpr int kBucketScatterIpt = 4;  // the scatter walks tiles of 4096 elements
 
 // Number of chunks a row-set is cut into.  Two per CU measured best from 2^24 to 2^28 keys:
 // long chunks keep the downsweep's pipeline and its carried partial lines busy (with one
 // tile per chunk every digit run starts and ends on a partial line), and the per-chunk
 // bookkeeping (one 256-entry count row, one start row) stays far below the key traffic.
-#ifndef MISORT_CHUNKS
-#define MISORT_CHUNKS 512
-#endif
-static constexpr size_t kTargetChunks  = MISORT_CHUNKS;
-#ifndef MISORT_SLAB
-#define MISORT_SLAB 16
-#endif
-static constexpr size_t kChunksPerSlab = MISORT_SLAB;
-#ifndef MISORT_UNT
-#define MISORT_UNT 256
-#endif
-static constexpr int kUpsweepThreads   = MISORT_UNT;
-#ifndef MISORT_UDT
-#define MISORT_UDT 256
-#endif
-static constexpr int kUpsweepDigitThreads = MISORT_UDT;  // upsweep over the digit side-band
+static constexpr size_t kTargetChunks  = 512;
+static constexpr size_t kChunksPerSlab = 16;
+static constexpr int kUpsweepThreads   = 256;
+static constexpr int kUpsweepDigitThreads = 256;  // upsweep over the digit side-band
 // values-only sorts of 2-byte elements: counted instead of radix-sorted from this length on
 static constexpr size_t kCount16MinLen = (size_t)1 << 20;
 static constexpr size_t kCount16Chunks = 512;
@@ -302,8 +355,9 @@ static constexpr size_t kCount16Chunks = 512;
 // target_chunks: chunks (workgroups) a radix pass over the whole array is cut into; 0 = the
 // built-in choice.  It is part of the plan, so the scratch query and the sort must agree on it.
 static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsort,
-                     bool has_indices_in, Plan& pl, size_t target_chunks = 0)
+                     bool has_indices_in, Plan& pl, const PlanOptions& opt = PlanOptions{})
 {
+  const size_t target_chunks = opt.target_chunks;
   if (!dtype_info(dtype, pl.dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
   pl.volume         = volume;
   pl.argsort        = argsort;
@@ -354,6 +408,24 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.has_indices_in    = true;
   }
 
+  if (pl.strategy == S_RADIX && pl.rows == 1 && pl.dt.bytes <= 8 && !pl.gather_values && opt.bucket_path != 0 &&
+      (opt.target_chunks == 0 || opt.bucket_path > 0)) {  // (a chunk count is a request to the radix path)
+    // One row of up to about a million elements: four launches in all instead of two per digit.
+    // The bins average a quarter of what the bin sort holds in registers (sample splitters:
+    // a bin four times the average does not happen), and there are at most 256 of them.
+    const size_t cap = opt.bucket_cap ? std::min<size_t>(opt.bucket_cap, (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay))
+                                      : (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay);
+    const size_t max_len = opt.bucket_path > 0 ? (size_t)0xFFFFFFFFu / 2 : 64 * cap;
+    if (pl.row_len <= max_len && cap >= 64) {
+      size_t bins = opt.bucket_bins ? opt.bucket_bins : (pl.row_len + 1023) / 1024;
+      if (bins < 2) bins = 2;
+      if (bins > 256) bins = 256;
+      pl.strategy = S_BUCKET;
+      pl.bk_split = (uint32_t)bins - 1;
+      pl.bk_cap   = (uint32_t)cap;
+    }
+  }
+
   size_t off = 0;
   auto take  = [&](size_t bytes) {
     const size_t o = off;
@@ -361,7 +433,21 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     return o;
   };
 
-  if (pl.strategy == S_RADIX) {
+  if (pl.strategy == S_BUCKET) {
+    pl.bk_tile            = BK_NT * kBucketScatterIpt;
+    const size_t tiles    = (pl.row_len + pl.bk_tile - 1) / pl.bk_tile;
+    const size_t want     = tiles < 256 ? tiles : 256;
+    pl.bk_tiles_per_chunk = (uint32_t)((tiles + want - 1) / want);
+    pl.bk_chunks          = (uint32_t)((tiles + pl.bk_tiles_per_chunk - 1) / pl.bk_tiles_per_chunk);
+    pl.bk_slabs           = (uint32_t)((pl.bk_chunks + kChunksPerSlab - 1) / kChunksPerSlab);
+    pl.off_bk_splitters   = take(BK_SLOTS * 8);
+    pl.off_bk_slab_tot    = take((size_t)pl.bk_slabs * BK_BINS * sizeof(uint32_t));
+    pl.off_bk_chunk_hist  = take((size_t)pl.bk_chunks * BK_BINS * sizeof(uint32_t));
+    pl.off_bk_bin_start   = take((BK_BINS + 1) * sizeof(uint32_t));
+    for (int b = 0; b < 2; ++b) pl.off_keys[b] = take(pl.volume * pl.dt.bytes);
+    if (pl.pay != PAY_NONE)
+      for (int b = 0; b < 2; ++b) pl.off_pay[b] = take(pl.volume * (pl.pay == PAY_IDX32 ? 4 : 8));
+  } else if (pl.strategy == S_RADIX) {
     pl.n_passes      = pl.dt.bytes;  // 8-bit digits
     pl.tile          = tile_size(pl.dt.bytes, pl.pay);
     pl.tiles_per_row = (pl.row_len + pl.tile - 1) / pl.tile;
@@ -378,6 +464,10 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     if (want < 1) want = 1;
     if (want > pl.tiles_per_row) want = pl.tiles_per_row;
     pl.tiles_per_chunk = (pl.tiles_per_row + want - 1) / want;
+    // a chunk's counts are 32-bit words (and the scatter multiplies the largest by 8): at most
+    // 2^29 keys per chunk, whatever the caller asked for
+    const size_t max_tpc = ((size_t)1 << 29) / (size_t)pl.tile;
+    if (pl.tiles_per_chunk > max_tpc) pl.tiles_per_chunk = max_tpc;
     pl.chunks_per_row  = (pl.tiles_per_row + pl.tiles_per_chunk - 1) / pl.tiles_per_chunk;
     pl.n_chunks        = pl.rows * pl.chunks_per_row;
     pl.chunks_per_slab = kChunksPerSlab;
@@ -419,7 +509,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // exponent, which vary in all but contrived inputs)
     pl.early_last =
       (pl.skip_dead_passes && (pl.dt.xform == XF_SIGNED || pl.dt.xform == XF_UNSIGNED) &&
-       pl.volume * pl.dt.bytes >= early_last_min_bytes())
+       pl.volume * pl.dt.bytes >= (opt.early_last_min_bytes >= 0 ? (size_t)opt.early_last_min_bytes
+                                                                       : early_last_min_bytes_default()))
         ? (int)pl.n_passes / 2
         : 0;
     pl.side_band = side_band_default() && pl.pay == PAY_NONE && pl.n_passes >= 2 && pl.dt.bytes == 8;
@@ -607,7 +698,7 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   pp.chunks_per_slab = (uint32_t)pl.chunks_per_slab;
   pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
   pp.xform           = pl.dt.xform;
-  pp.rank_by_add     = rank_by_add_default();
+  pp.rank_by_add     = rank_by_add_on_current_device();
   pp.n_rows          = (uint32_t)pl.rows;
   pp.key_buf[0]      = S + pl.off_keys[0];
   pp.key_buf[1]      = S + pl.off_keys[1];
@@ -755,6 +846,77 @@ static void radix_sort_dispatch(Launcher& L, const Plan& pl, const SortArgs& a)
 }
 
 // ---------------------------------------------------------------------------------------
+// one row through sample -> count -> scatter -> sort the bins (bucket.hpp)
+// ---------------------------------------------------------------------------------------
+template <typename KeyT, int PAY>
+static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a)
+{
+  char* S = a.scratch;
+  BucketParams p{};
+  p.keys_in         = a.values_in;
+  p.pay_in          = a.indices_in;
+  p.keys_out        = a.values_out;
+  p.pay_out         = a.indices_out;
+  p.buf_keys[0]     = S + pl.off_keys[0];
+  p.buf_keys[1]     = S + pl.off_keys[1];
+  p.buf_pay[0]      = PAY != PAY_NONE ? S + pl.off_pay[0] : nullptr;
+  p.buf_pay[1]      = PAY != PAY_NONE ? S + pl.off_pay[1] : nullptr;
+  p.splitters       = S + pl.off_bk_splitters;
+  p.slab_tot        = reinterpret_cast<uint32_t*>(S + pl.off_bk_slab_tot);
+  p.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_bk_chunk_hist);
+  p.bin_start       = reinterpret_cast<uint32_t*>(S + pl.off_bk_bin_start);
+  p.n               = (uint32_t)pl.row_len;
+  p.n_split         = pl.bk_split;
+  p.tile            = pl.bk_tile;
+  p.tiles_per_chunk = pl.bk_tiles_per_chunk;
+  p.n_chunks        = pl.bk_chunks;
+  p.chunks_per_slab = (uint32_t)kChunksPerSlab;
+  p.n_slabs         = pl.bk_slabs;
+  p.cap             = pl.bk_cap;
+  p.index_offset    = a.index_offset;
+  p.xform           = pl.dt.xform;
+  p.keys_travel     = pl.dt.xform == XF_COMPLEX ? 1 : 0;
+  p.rank_by_add     = rank_by_add_on_current_device();
+  p.dbg_max_bits    = getenv("DBG_MAX_BITS") ? atoi(getenv("DBG_MAX_BITS")) : -1;
+  p.direct_equal    = (a.values_out == nullptr || a.values_out != a.values_in) &&
+                      (a.indices_out == nullptr || a.indices_out != a.indices_in);
+  constexpr int IPT = bucket_sort_ipt(sizeof(KeyT), PAY);
+  L.run(K_BUCKET_PLAN, [&] {
+    hipLaunchKernelGGL((bucket_plan_kernel<KeyT>), dim3(1), dim3(BK_PLAN_NT), 0, L.stream, p);
+  });
+  L.run(K_BUCKET_COUNT, [&] {
+    hipLaunchKernelGGL((bucket_count_kernel<KeyT>), dim3(pl.bk_chunks), dim3(BK_COUNT_NT), 0, L.stream, p);
+  });
+  L.run(K_BUCKET_SCATTER, [&] {
+    hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, kBucketScatterIpt>), dim3(pl.bk_chunks), dim3(BK_NT), 0,
+                       L.stream, p);
+  });
+  L.run(K_BUCKET_SORT, [&] {
+    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(pl.bk_split + 1), dim3(BK_NT), 0, L.stream, p);
+  });
+}
+
+template <typename KeyT>
+static void bucket_sort_dispatch_pay(Launcher& L, const Plan& pl, const SortArgs& a)
+{
+  switch (pl.pay) {
+    case PAY_NONE: bucket_sort_row<KeyT, PAY_NONE>(L, pl, a); break;
+    case PAY_IDX32: bucket_sort_row<KeyT, PAY_IDX32>(L, pl, a); break;
+    default: bucket_sort_row<KeyT, PAY_I64>(L, pl, a); break;
+  }
+}
+
+static void bucket_sort_dispatch(Launcher& L, const Plan& pl, const SortArgs& a)
+{
+  switch (pl.dt.bytes) {
+    case 1: bucket_sort_dispatch_pay<uint8_t>(L, pl, a); break;
+    case 2: bucket_sort_dispatch_pay<uint16_t>(L, pl, a); break;
+    case 4: bucket_sort_dispatch_pay<uint32_t>(L, pl, a); break;
+    default: bucket_sort_dispatch_pay<uint64_t>(L, pl, a); break;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // counting sort of one long row of 2-byte elements (values only)
 // ---------------------------------------------------------------------------------------
 static void count16_sort(Launcher& L, const Plan& pl, const SortArgs& a)
@@ -855,7 +1017,10 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
 {
   DtypeInfo dt;
   if (!dtype_info(dtype, dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
-  int rc = make_plan(dtype, volume, sort_dim_size, want_indices, false, u.pl);
+  // (the selection walks the chunks of the radix plan)
+  PlanOptions radix_only;
+  radix_only.bucket_path = 0;
+  int rc = make_plan(dtype, volume, sort_dim_size, want_indices, false, u.pl, radix_only);
   if (rc != MISORT_OK) return rc;
   // 1- and 2-byte values are counted, which beats selecting; their positions are selected
   u.select = u.pl.strategy == S_RADIX && u.pl.pay != PAY_I64 && kth >= 0 &&
@@ -886,7 +1051,7 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   u.off_pass_hist   = take((size_t)dt.bytes * pl.n_chunks * RADIX * sizeof(uint32_t));
   u.off_sel_state   = take(pl.rows * sizeof(uint32_t));
   u.off_n_equal     = take(pl.rows * sizeof(unsigned long long));
-  u.off_above_max   = take(pl.rows * 2 * sizeof(unsigned long long));
+  u.off_above_max   = take(pl.rows * 3 * sizeof(unsigned long long));
   u.off_cand_from   = take(pl.rows * sizeof(uint32_t));
   u.off_cand_n      = take(pl.rows * sizeof(unsigned long long));
   u.cand_cap        = pl.row_len / 8 + 1;  // keys that still match, once they are this few
@@ -1003,11 +1168,11 @@ static void select_rows(Launcher& L, const PartLayout& u, const void* vin, long 
 static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_out,
                     const int64_t* indices_in, int64_t* indices_out, size_t volume,
                     size_t sort_dim_size, int64_t index_offset, void* scratch, size_t scratch_bytes,
-                    size_t target_chunks = 0, bool canonical_values = false)
+                    const PlanOptions& opt = PlanOptions{}, bool canonical_values = false)
 {
   Plan pl;
   const bool argsort = indices_out != nullptr;
-  int rc = make_plan(dtype, volume, sort_dim_size, argsort, indices_in != nullptr, pl, target_chunks);
+  int rc = make_plan(dtype, volume, sort_dim_size, argsort, indices_in != nullptr, pl, opt);
   if (rc != MISORT_OK) return rc;
   if (pl.strategy == S_EMPTY) return MISORT_OK;
 
@@ -1074,6 +1239,7 @@ static int run_sort(Launcher& L, int dtype, const void* values_in, void* values_
       break;
     case S_COUNT16: count16_sort(L, pl, core); break;
     case S_COUNT8: count8_sort(L, pl, core); break;
+    case S_BUCKET: bucket_sort_dispatch(L, pl, core); break;
     case S_RADIX:
       radix_sort_dispatch(L, pl, core);
       if (pl.gather_values) {
@@ -1109,17 +1275,24 @@ static __device__ __align__(256) unsigned char misort_static_scratch[MISORT_STAT
 
 namespace misort {
 
-static constexpr int kMaxDevices = 64;
 static std::atomic<void*> g_static_scratch_ptr[kMaxDevices];
 
-// Device address of misort_static_scratch on the current GPU, looked up once per GPU.
-static int static_scratch_address(void** out)
+// Device address of misort_static_scratch on the current GPU, looked up once per GPU.  A
+// stream that belongs to another GPU than the current one is refused: its kernels would be
+// handed the current GPU's copy of the buffer.
+static int static_scratch_address(void** out, hipStream_t stream = nullptr)
 {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess)
     return fail(MISORT_ERR_RUNTIME, std::string("hipGetDevice: ") + hipGetErrorString(e));
   if (dev < 0 || dev >= kMaxDevices) return fail(MISORT_ERR_UNSUPPORTED, "device ordinal above 63");
+  if (stream) {
+    hipDevice_t sdev = -1;
+    if (hipStreamGetDevice(stream, &sdev) == hipSuccess && (int)sdev != dev)
+      return fail(MISORT_ERR_UNSUPPORTED, "misort_local_static: the stream belongs to another GPU than the current one");
+    (void)hipGetLastError();
+  }
   void* p = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
   if (!p) {
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(misort_static_scratch));
@@ -1183,7 +1356,7 @@ int misort_local_static(int dtype, const void* values_in, void* values_out, cons
   }
   if (pl.strategy == S_EMPTY) return MISORT_OK;
   void* own = nullptr;
-  rc        = static_scratch_address(&own);
+  rc        = static_scratch_address(&own, reinterpret_cast<hipStream_t>(stream));
   if (rc != MISORT_OK) return rc;
   Launcher L;
   L.stream = reinterpret_cast<hipStream_t>(stream);
@@ -1195,8 +1368,9 @@ size_t misort_scratch_bytes_chunked(int dtype, size_t volume, size_t sort_dim_si
                                     int has_indices_in, size_t target_chunks)
 {
   Plan pl;
-  if (make_plan(dtype, volume, sort_dim_size, argsort != 0, has_indices_in != 0, pl, target_chunks) !=
-      MISORT_OK)
+  PlanOptions opt;
+  opt.target_chunks = target_chunks;
+  if (make_plan(dtype, volume, sort_dim_size, argsort != 0, has_indices_in != 0, pl, opt) != MISORT_OK)
     return 0;
   return pl.total;
 }
@@ -1208,8 +1382,61 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
 {
   Launcher L;
   L.stream = reinterpret_cast<hipStream_t>(stream);
+  PlanOptions opt;
+  opt.target_chunks = target_chunks;
   return run_sort(L, dtype, values_in, values_out, indices_in, indices_out, volume, sort_dim_size,
-                  index_offset, scratch, scratch_bytes, target_chunks);
+                  index_offset, scratch, scratch_bytes, opt);
+}
+
+static PlanOptions plan_options(const misort_options* o)
+{
+  PlanOptions opt;
+  if (o) {
+    opt.target_chunks        = o->target_chunks;
+    opt.early_last_min_bytes = o->early_last_min_bytes;
+    opt.bucket_path          = o->bucket_path;
+    opt.bucket_bins          = o->bucket_bins;
+    opt.bucket_cap           = o->bucket_cap;
+  }
+  return opt;
+}
+
+size_t misort_scratch_bytes_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
+                                 int has_indices_in, const misort_options* options)
+{
+  Plan pl;
+  if (make_plan(dtype, volume, sort_dim_size, argsort != 0, has_indices_in != 0, pl, plan_options(options)) !=
+      MISORT_OK)
+    return 0;
+  return pl.total;
+}
+
+int misort_local_opts(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
+                      int64_t* indices_out, size_t volume, size_t sort_dim_size, int /*stable*/,
+                      int64_t index_offset, void* scratch, size_t scratch_bytes, void* stream,
+                      const misort_options* options)
+{
+  Launcher L;
+  L.stream = reinterpret_cast<hipStream_t>(stream);
+  return run_sort(L, dtype, values_in, values_out, indices_in, indices_out, volume, sort_dim_size,
+                  index_offset, scratch, scratch_bytes, plan_options(options));
+}
+
+int misort_init(void)
+{
+  void* own = nullptr;
+  const int rc = static_scratch_address(&own);
+  if (rc != MISORT_OK) return rc;
+  (void)rank_by_add_on_current_device();
+  return MISORT_OK;
+}
+
+int misort_rank_mode(void)
+{
+  if (rank_ballot_env()) return 2;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  return g_rank_mode[dev].load(std::memory_order_acquire);
 }
 
 int misort_local_profiled(int dtype, const void* values_in, void* values_out,
@@ -1249,11 +1476,20 @@ const char* misort_kernel_name(int kernel_id)
 int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                          int has_indices_in, char* buf, size_t buf_bytes)
 {
+  return misort_describe_plan_opts(dtype, volume, sort_dim_size, argsort, has_indices_in, nullptr, buf,
+                                   buf_bytes);
+}
+
+int misort_describe_plan_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
+                              int has_indices_in, const misort_options* options, char* buf,
+                              size_t buf_bytes)
+{
   Plan pl;
-  const int rc = make_plan(dtype, volume, sort_dim_size, argsort != 0, has_indices_in != 0, pl);
+  const int rc =
+    make_plan(dtype, volume, sort_dim_size, argsort != 0, has_indices_in != 0, pl, plan_options(options));
   if (rc != MISORT_OK) return rc;
   if (!buf || buf_bytes == 0) return fail(MISORT_ERR_NULL, "buf is NULL");
-  static const char* const sname[] = {"empty", "row_wave", "row_block", "radix", "count16", "count8"};
+  static const char* const sname[] = {"empty", "row_wave", "row_block", "radix", "count16", "count8", "bucket"};
   static const char* const pname[] = {"none", "idx32", "i64"};
   snprintf(buf, buf_bytes,
            "strategy=%s key_bytes=%d passes=%d digit_bits=%d tile=%d rows=%zu row_len=%zu "
@@ -1262,10 +1498,21 @@ int misort_describe_plan(int dtype, size_t volume, size_t sort_dim_size, int arg
            sname[pl.strategy], pl.dt.bytes, pl.n_passes, RADIX_BITS, pl.tile, pl.rows, pl.row_len,
            pl.chunks_per_row, pl.tiles_per_chunk, pname[pl.pay], (int)pl.specials,
            (int)pl.gather_values, pl.side_band ? 1 : (pl.side_adaptive ? 2 : 0), pl.total);
+  if (pl.strategy == S_BUCKET) {
+    const size_t len = strlen(buf);
+    if (len + 64 < buf_bytes)
+      snprintf(buf + len, buf_bytes - len, " bins=%u bin_cap=%u chunks=%u", pl.bk_split + 1, pl.bk_cap, pl.bk_chunks);
+  }
   if (pl.skip_dead_passes) {
     const size_t len = strlen(buf);
     if (len + 32 < buf_bytes)
       snprintf(buf + len, buf_bytes - len, " skip_dead_passes=1%s", pl.early_last ? " early_last=1" : "");
+  }
+  if (pl.strategy == S_RADIX || pl.strategy == S_BUCKET) {
+    // how the scatter ranks on the current GPU (decided at the first sort there or by misort_init)
+    static const char* const rname[] = {"untested", "add", "ballot"};
+    const size_t len = strlen(buf);
+    if (len + 16 < buf_bytes) snprintf(buf + len, buf_bytes - len, " rank=%s", rname[misort_rank_mode()]);
   }
   return MISORT_OK;
 }
@@ -1325,7 +1572,7 @@ int misort_searchsorted_ws(int dtype, const void* sorted, size_t n, const void* 
     char* S      = reinterpret_cast<char*>(scratch);
     int64_t* pos = reinterpret_cast<int64_t*>(S + u.off_pos);
     const int rc = run_sort(L, dtype, values, S, nullptr, pos, m, m, 0, S + u.off_sort,
-                            u.sort_bytes > 0 ? u.sort_bytes : 256, 0, true);
+                            u.sort_bytes > 0 ? u.sort_bytes : 256, PlanOptions{}, true);
     if (rc != MISORT_OK) return rc;
     queries = S;
     where   = pos;
@@ -1616,6 +1863,7 @@ int misort_selftest_lds_lane_order(unsigned int rows_per_wave, unsigned long lon
                                    unsigned long long* out_of_order, void* stream)
 {
   if (!checked || !out_of_order) return fail(MISORT_ERR_NULL, "selftest: NULL pointer");
+  std::lock_guard<std::mutex> lock(g_probe_mutex);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   unsigned long long* counts = nullptr;
   hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&counts), HIP_SYMBOL(g_selftest_counts));

@@ -220,10 +220,7 @@ __device__ __forceinline__ void pin_value(T& v)
 // A pass without a byte carry writes the digit side-band only if a tile of the row holds at
 // most this many digit values on average (random digits: 256, where it costs 0.4 ms per pass
 // at 2^28 keys and saves 0.15-0.3 ms in the next upsweep).
-#ifndef MISORT_SIDE_PRESENT_MAX
-#define MISORT_SIDE_PRESENT_MAX 64
-#endif
-static constexpr uint32_t kSidePresentMax = MISORT_SIDE_PRESENT_MAX;
+static constexpr uint32_t kSidePresentMax = 64;
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load and store of the wave, which would serialise the prefetch of the

@@ -74,7 +74,9 @@ struct SelectParams {
   unsigned long long* cand_n;     // per row: candidates written
   uint64_t cand_cap;
   unsigned long long* n_equal;    // per row: keys equal to the kth key (known after the last pick)
-  unsigned long long* above_max;  // per row: smallest key above the kth key, largest key (misort_select only)
+  unsigned long long* above_max;  // per row, three words (misort_select only): smallest key above the kth
+                                 // key among the candidates, largest key of the row, smallest key above
+                                 // the kth key found by the read of the row itself
   uint32_t* cand_less_eq;         // per chunk: candidates below the kth key, and equal to it
   // for the split pass
   uint32_t* chunk_cls;            // [chunk][4]: keys below / equal to / above the kth key (and a pad)
@@ -196,7 +198,7 @@ __global__ void __launch_bounds__(SEL_NT) select_hist_kernel(SelectParams<KeyT> 
           const unsigned long long h2 = __shfl_xor(hi, s, 64);
           hi = h2 > hi ? h2 : hi;
         }
-        if (lane == 0 && b1 > b0) atomicMax(&p.above_max[2 * (uint64_t)row + 1], hi);
+        if (lane == 0 && b1 > b0) atomicMax(&p.above_max[3 * (uint64_t)row + 1], hi);
       }
     }
   };
@@ -261,8 +263,9 @@ __global__ void __launch_bounds__(256) select_init_kernel(SelectParams<KeyT> p, 
     p.cand_from[r] = p.n_passes;
     p.cand_n[r]    = 0;
     if (p.above_max) {
-      p.above_max[2 * (uint64_t)r]     = ~0ull;
-      p.above_max[2 * (uint64_t)r + 1] = 0;
+      p.above_max[3 * (uint64_t)r]     = ~0ull;
+      p.above_max[3 * (uint64_t)r + 1] = 0;
+      p.above_max[3 * (uint64_t)r + 2] = ~0ull;
     }
   }
 }
@@ -505,11 +508,13 @@ select_split_kernel(SelectParams<KeyT> p, KeyT* __restrict__ values_out, int64_t
 
 // grid: n_chunks, after the last pick; keys of at most 8 bytes.  For callers that want the
 // key after the kth one instead of a partitioned row: the smallest key above the kth key,
-// into above_max[2 * row] (all ones on entry).  Run twice: with CAND over the candidates of
-// the rows that have some (the key is nearly always among them), then without over the rows
-// themselves, where the workgroups of a row leave at once unless the answer is still open:
-// as many keys equal the kth key as lie at or before kth, and the candidates had nothing
-// above it.  (The largest key of the row, the other word, comes from the first histogram pass.)
+// (all ones where there is none).  Run twice: with CAND over the candidates of the rows that
+// have some (the key is nearly always among them; into word 0 of the row's three), then
+// without over the rows themselves (into word 2), where the workgroups of a row leave at once
+// unless the answer is still open: as many keys equal the kth key as lie at or before kth,
+// and the candidates had nothing above it.  The second launch decides that from word 0 alone,
+// which only the first launch writes: a word that its own workgroups update could send a
+// workgroup that starts late away from a chunk that holds the answer.  (The largest key of the row, the other word, comes from the first histogram pass.)
 template <typename KeyT, bool CAND>
 __global__ void __launch_bounds__(SEL_NT) select_above_kernel(SelectParams<KeyT> p)
 {
@@ -529,8 +534,9 @@ __global__ void __launch_bounds__(SEL_NT) select_above_kernel(SelectParams<KeyT>
     b0   = (uint64_t)chunk * per;
     b1   = b0 + per < n_c ? b0 + per : n_c;
   } else {
-    // (plain loads of a word that atomics of the launch before wrote: that launch is complete)
-    if (p.above_max[2 * (uint64_t)row] != ~0ull) return;
+    // (plain loads of a word that atomics of the launch before wrote: that launch is complete,
+    // and this launch writes word 2 only)
+    if (p.above_max[3 * (uint64_t)row] != ~0ull) return;
     base = p.in + (uint64_t)row * p.row_len;
     b0   = (uint64_t)chunk * p.chunk_len;
     b1   = b0 + p.chunk_len;
@@ -568,7 +574,7 @@ __global__ void __launch_bounds__(SEL_NT) select_above_kernel(SelectParams<KeyT>
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < SEL_NT / 64; ++w) lo = wmin[w] < lo ? wmin[w] : lo;
-    if (lo != ~0ull) atomicMin(&p.above_max[2 * (uint64_t)row], lo);
+    if (lo != ~0ull) atomicMin(&p.above_max[3 * (uint64_t)row + (CAND ? 0 : 2)], lo);
   }
 }
 
@@ -583,8 +589,9 @@ select_emit_kernel(SelectParams<KeyT> p, uint32_t rows, KeyT* __restrict__ kth_o
 {
   for (uint32_t r = blockIdx.x * 256 + threadIdx.x; r < rows; r += gridDim.x * 256) {
     const KeyT kth  = p.prefix[r];
-    const KeyT top  = (KeyT)p.above_max[2 * (uint64_t)r + 1];
-    KeyT above      = (KeyT)p.above_max[2 * (uint64_t)r];
+    const KeyT top  = (KeyT)p.above_max[3 * (uint64_t)r + 1];
+    const unsigned long long a0 = p.above_max[3 * (uint64_t)r], a2 = p.above_max[3 * (uint64_t)r + 2];
+    KeyT above      = (KeyT)(a0 < a2 ? a0 : a2);
     if (above > top) above = top;  // nothing above: the row ends at kth (callers do not ask then)
     if (kth_out) kth_out[r] = KeyOps<KeyT>::from_key(kth, p.xform);
     if (next_out) next_out[r] = KeyOps<KeyT>::from_key(p.kleft[r] + 1 < p.n_equal[r] ? kth : above, p.xform);

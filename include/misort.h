@@ -23,9 +23,10 @@
 extern "C" {
 #endif
 
-/* Element type codes.  Values follow legate's Type::Code numbering, which is
- * also the order of cuNumeric's SUPPORTED_DTYPES table (reference:
- * cunumeric/utils.py:29-44). */
+/* Element type codes, in the order of cuNumeric's SUPPORTED_DTYPES table (reference:
+ * cunumeric/utils.py:29-44).  They are this library's own numbers: a binding maps its
+ * framework's type enumeration to them by name (INTEGRATION.md shows the switch), never by
+ * casting one enumeration to the other. */
 typedef enum misort_dtype {
   MISORT_BOOL       = 0,
   MISORT_INT8       = 1,
@@ -82,7 +83,8 @@ const char* misort_last_error(void);
  * Radix passes over a digit that is the same in every key are skipped (decided on the device,
  * nothing is read back); MISORT_SKIP_PASSES=0 runs them all.  Sorts of 256 MB of keys and
  * more also leave out the passes over constant most significant digits (the last pass whose
- * digit varies writes the result); MISORT_EARLY_LAST_BYTES=<bytes> moves that limit.
+ * digit varies writes the result); MISORT_EARLY_LAST_BYTES=<bytes> moves that limit.  All
+ * four variables are read once, when the library is first used.
  */
 size_t misort_scratch_bytes(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                             int has_indices_in);
@@ -244,17 +246,78 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
                          size_t target_chunks);
 
 /*
+ * misort_scratch_bytes / misort_local with choices that are otherwise built in, per call (a
+ * NULL pointer or a zeroed struct with early_last_min_bytes = bucket_path = -1 means "as
+ * misort_local").  No counterpart in the reference; for tests that have to reach the code for
+ * large or unusual inputs with small arrays, and for measurements.  Give the query and the
+ * sort the same options.
+ *   target_chunks         as misort_local_chunked (0: built in)
+ *   early_last_min_bytes  from how many bytes of keys on the passes over constant most
+ *                         significant digits are left out as well (< 0: built in, 256 MB)
+ *   bucket_path           single rows of up to about a million elements are sorted in four
+ *                         launches (splitters from a sorted sample, count, scatter into at most
+ *                         256 bins, radix sort of every bin inside one workgroup) instead of two
+ *                         launches per digit.  < 0: built in; 0: never; > 0: for every single
+ *                         row of 1- to 8-byte elements, whatever its length
+ *   bucket_bins           number of bins, 2 .. 256 (0: built in, one per 1024 elements)
+ *   bucket_cap            longest bin that is sorted in registers; longer ones take the
+ *                         workgroup's loop through global memory (0: built in, 8192 or 16384)
+ */
+typedef struct misort_options {
+  size_t target_chunks;
+  long long early_last_min_bytes;
+  int bucket_path;
+  unsigned bucket_bins;
+  unsigned bucket_cap;
+} misort_options;
+size_t misort_scratch_bytes_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
+                                 int has_indices_in, const misort_options* options);
+int misort_local_opts(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
+                      int64_t* indices_out, size_t volume, size_t sort_dim_size, int stable,
+                      int64_t index_offset, void* scratch, size_t scratch_bytes, void* stream,
+                      const misort_options* options);
+/* misort_describe_plan for the plan that misort_local_opts would execute with `options`. */
+int misort_describe_plan_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
+                              int has_indices_in, const misort_options* options, char* buf,
+                              size_t buf_bytes);
+
+/*
+ * One-time set-up for the GPU that is current on the calling thread, optional: looks up the
+ * address of the library's own scratch buffer (misort_local_static) and decides how the radix
+ * scatter ranks on this GPU (misort_rank_mode).  Both happen by themselves in the first call
+ * that needs them; a caller that records its calls into a HIP graph, or must not see a
+ * synchronisation later, calls this first, outside any capture.  No counterpart in the
+ * reference (static registration, src/cunumeric/sort/sort.cc:73-81, is the nearest thing).
+ */
+int misort_init(void);
+
+/*
+ * How the radix scatter ranks the keys of a wavefront on the current GPU: 1 = one returning
+ * LDS add per key, 2 = wave ballots, 0 = not decided yet (no sort has run here and
+ * misort_init was not called).  The adds are stable only where the LDS serves the lanes of
+ * one instruction that hit the same word in ascending lane order; the library uses them only
+ * on gfx950 and only after a probe of 25 million lane operations on that GPU (about 0.1 ms,
+ * on a stream of its own, once per GPU and process) has found every lane in order, and
+ * MISORT_RANK_BALLOT=1 in the environment rules them out.  No counterpart in the reference.
+ */
+int misort_rank_mode(void);
+
+/*
  * misort_local without a scratch argument and without any allocation: the scratch is a
  * buffer of MISORT_STATIC_SCRATCH_BYTES that the library itself holds in device memory on
  * every GPU it runs on, until the process ends.  No counterpart in the reference (which
  * allocates from the Legate pool in every call, src/cunumeric/sort/cub_sort.cuh:46-62); it is
- * for callers that cannot allocate: code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc.  Same arguments and results as misort_local.  A sort
+ * for callers that cannot allocate: tight serving loops, harnesses that forbid hipMalloc, code
+ * that records into a HIP graph (call misort_init before the capture starts: the first call
+ * on a GPU looks the buffer's address up and probes the LDS, neither of which may be
+ * recorded).  Same arguments and results as misort_local.  A sort
  * whose misort_scratch_bytes exceeds MISORT_STATIC_SCRATCH_BYTES is refused with
  * MISORT_ERR_SCRATCH (nothing is launched).  All calls on one GPU share the one buffer:
  * calls that overlap in time on the same GPU (different streams or threads) race; calls
  * ordered on one stream are safe.  The first call on a GPU looks the buffer's address up
  * (hipGetSymbolAddress); no call uses hipMalloc, hipFree or an allocating library routine.
+ * `stream` must belong to the GPU that is current on the calling thread (each GPU has its own
+ * copy of the buffer); a stream of another GPU is refused with MISORT_ERR_UNSUPPORTED.
  */
 #define MISORT_STATIC_SCRATCH_BYTES (64u << 20)
 int misort_local_static(int dtype, const void* values_in, void* values_out, const int64_t* indices_in,
@@ -269,8 +332,9 @@ int misort_local_static(int dtype, const void* values_in, void* values_out, cons
  * rows_per_wave instructions with few distinct addresses, every lane compared with its rank
  * by the ballot match.  *checked receives the number of lanes compared, *out_of_order the
  * number that disagreed (0 on every MI355X seen).  Host pointers; synchronises `stream`.
- * Setting MISORT_RANK_BALLOT=1 in the environment before the first call into the library
- * makes every sort rank by ballots instead.
+ * The library runs a short form of the same probe by itself before it first uses the adds on a
+ * GPU (misort_rank_mode); setting MISORT_RANK_BALLOT=1 in the environment before the first
+ * call into the library makes every sort rank by ballots instead.
  */
 int misort_selftest_lds_lane_order(unsigned int rows_per_wave, unsigned long long* checked,
                                    unsigned long long* out_of_order, void* stream);

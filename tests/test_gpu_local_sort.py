@@ -10,9 +10,13 @@ from tests.util import ALL_DTYPES, Abi, bits_equal, random_array
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def abi():
-    return Abi()
+@pytest.fixture(scope="module", params=[False, True], ids=["default plan", "radix path asked for"])
+def abi(request):
+    # single rows of 16385 to about a million elements take the four-launch path by default;
+    # the second round runs the same cases on the radix path, which serves the longer rows
+    a = Abi()
+    a.force_radix = request.param
+    return a
 
 
 SIZES_1D = [1, 2, 63, 64, 65, 255, 500, 513, 1000, 1024, 1025, 4096, 4097, 8192, 8193, 12289, 100003]

@@ -15,9 +15,13 @@ ROW_LENGTHS = [1, 5, 33, 64, 200, 1024, 1025, 3000, 4096, 8192, 8193, 16384, 163
                150000, 400000]
 
 
-@pytest.fixture(scope="module")
-def abi():
-    return Abi()
+@pytest.fixture(scope="module", params=[False, True], ids=["default plan", "radix path asked for"])
+def abi(request):
+    # single rows of 16385 to about a million elements take the four-launch path by default;
+    # the second round runs the same cases on the radix path, which serves the longer rows
+    a = Abi()
+    a.force_radix = request.param
+    return a
 
 
 def draw(rng, dtype, total, kind):
@@ -40,7 +44,7 @@ def same_bits_or_values(got, ref):
 
 
 @pytest.mark.parametrize("seed", range(4))
-def test_random_calls(abi, seed, monkeypatch):
+def test_random_calls(abi, seed):
     rng = np.random.default_rng(2000 + seed)
     for it in range(150):
         dtype = ALL_DTYPES[rng.integers(0, len(ALL_DTYPES))]
@@ -74,7 +78,8 @@ def test_random_calls(abi, seed, monkeypatch):
             assert np.array_equal(gi.reshape(rows, row), perm + off), tag
             assert same_bits_or_values(gv.reshape(rows, row), s), tag
         else:            # the early last pass on for every size, or for none
-            monkeypatch.setenv("MISORT_EARLY_LAST_BYTES", str(int(rng.choice([0, 1 << 40]))))
-            got = abi.local_sort(a, row, argsort=True, **kw).reshape(rows, row)
-            monkeypatch.delenv("MISORT_EARLY_LAST_BYTES")
+            if static:
+                kw = dict(chunks=chunks)
+            got = abi.local_sort(a, row, argsort=True, early_last_bytes=int(rng.choice([0, 1 << 40])),
+                                 **kw).reshape(rows, row)
             assert np.array_equal(got, perm), tag

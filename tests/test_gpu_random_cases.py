@@ -4,8 +4,7 @@ stable sort), sort (bit-exact) and stable argsort (exact), over element types, r
 row lengths off every alignment and key distributions that steer the kernels differently:
 full range, few values, pools of repeated values (runs of equal keys in the later passes),
 small ranges (dead leading bytes), sorted input, one value holding most of the row, small values
-of both signs.  Half of the seeds also let small sorts leave out constant leading digits
-(MISORT_EARLY_LAST_BYTES=0), which large sorts do by themselves."""
+of both signs."""
 import numpy as np
 import pytest
 
@@ -46,11 +45,7 @@ def draw(rng, dtype, rows, n, kind):
 
 
 @pytest.mark.parametrize("seed", range(6))
-def test_random_cases(seed, monkeypatch):
-    if seed % 2:
-        monkeypatch.setenv("MISORT_EARLY_LAST_BYTES", "0")
-    else:
-        monkeypatch.delenv("MISORT_EARLY_LAST_BYTES", raising=False)
+def test_random_cases(seed):
     abi = Abi()
     rng = np.random.default_rng(1000 + seed)
     for it in range(12):

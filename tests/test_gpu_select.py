@@ -122,6 +122,27 @@ def test_next_element_lies_outside_the_keys_that_still_match(abi, dtype):
         assert same_values(k, s[:, kth]) and same_values(nxt, s[:, kth + 1]) and same_values(top, s[:, -1]), kth
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.uint64], ids=lambda d: np.dtype(d).name)
+def test_next_element_held_by_one_chunk_of_a_row_without_candidates(abi, dtype):
+    """Rows of one repeated value plus a few larger ones: the keys that still match never
+    become few enough to be written out, so the element after kth comes from the read of the
+    row itself, and here the smallest larger value sits in the last chunk only while the
+    first chunk holds a larger one.  Every workgroup of the row has to look at its chunk,
+    whatever the others have already reported."""
+    n = 600007
+    for rep in range(3):
+        a = np.full((2, n), 5, dtype=dtype)
+        a[0, 3] = 900
+        a[0, n - 2 - rep] = 7      # the answer, in the last chunk
+        a[1, n - 5] = 901
+        a[1, 11 + rep] = 8         # the answer, in the first chunk
+        a[1, n // 2] = 4
+        s = np.sort(a, axis=1)
+        for kth in (n - 3, n - 4, 0):
+            k, nxt, top = select(abi, a, kth)
+            assert same_values(k, s[:, kth]) and same_values(nxt, s[:, kth + 1]) and same_values(top, s[:, -1]), kth
+
+
 def test_nan_rows_and_signed_zeros(abi):
     rng = np.random.default_rng(63)
     n = 70001

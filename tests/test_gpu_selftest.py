@@ -37,6 +37,8 @@ import numpy as np, sys
 sys.path.insert(0, %r)
 from tests.util import Abi, random_array
 abi = Abi()
+abi.force_radix = True
+assert abi.lib.misort_rank_mode() == 2
 rng = np.random.default_rng(5)
 for dtype, n in ((np.float32, 300001), (np.int64, 200003), (np.uint32, 1 << 20)):
     a = random_array(dtype, n, rng)

@@ -17,7 +17,9 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(scope="module")
 def abi():
-    return Abi()
+    a = Abi()
+    a.force_radix = True  # (single rows of this length would take the four-launch path otherwise)
+    return a
 
 
 def cases(dtype, n, rng):
@@ -78,6 +80,7 @@ def test_switch_off_gives_the_same_result():
         "rng = np.random.default_rng(44)\n"
         "a = rng.standard_normal(300001)\n"
         "abi = Abi()\n"
+        "abi.force_radix = True\n"
         "plan = abi.describe_plan(np.float64, a.size, a.size, False)\n"
         "s = abi.local_sort(a, a.size, argsort=False, chunks=3)\n"
         "sys.stdout.write(plan + '\\n' + str(bool((s == np.sort(a)).all())) + '\\n')\n"

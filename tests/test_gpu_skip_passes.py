@@ -2,8 +2,9 @@
 first upsweep ORs the keys and their complements; every later kernel derives from those
 words which passes are dead and which ping-pong buffer holds its input).  Large sorts also
 leave out the passes over the most significant digits if those are constant: the last pass
-whose digit varies then writes the result; MISORT_EARLY_LAST_BYTES=0 makes small sorts do
-the same, which is how the tests below reach that path.  Inputs whose
+whose digit varies then writes the result; early_last_min_bytes = 0 in the options of
+misort_local_opts makes small sorts do the same, which is how the tests below reach that path
+(they also ask for the radix path, which single rows of this length no longer take by themselves).  Inputs whose
 constant bytes sit in every combination of positions, for all key widths with middle passes,
 sorts and argsorts, rows, a caller payload, and the same input with the skipping switched
 off must agree with NumPy."""
@@ -21,16 +22,16 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(scope="module")
 def abi():
-    return Abi()
+    a = Abi()
+    a.force_radix = True
+    return a
 
 
 @pytest.fixture(params=[False, True], ids=["top pass kept", "last live pass writes the result"])
-def early_last(request, monkeypatch):
-    if request.param:
-        monkeypatch.setenv("MISORT_EARLY_LAST_BYTES", "0")
-    else:
-        monkeypatch.delenv("MISORT_EARLY_LAST_BYTES", raising=False)
-    return request.param
+def early_last(request, abi):
+    abi.early_last_bytes = 0 if request.param else 1 << 40
+    yield request.param
+    abi.early_last_bytes = None
 
 
 def masked_random(dtype, n, rng, live_bytes):
@@ -159,6 +160,7 @@ def test_switch_off_gives_the_same_result():
         "rng = np.random.default_rng(64)\n"
         "a = rng.integers(0, 300, 400001, dtype=np.int64)\n"
         "abi = Abi()\n"
+        "abi.force_radix = True\n"
         "plan = abi.describe_plan(np.int64, a.size, a.size, True)\n"
         "s = abi.local_sort(a, a.size, argsort=True, chunks=3)\n"
         "sys.stdout.write(plan + '\\n' + str(bool((s == np.argsort(a, kind='stable')).all())) + '\\n')\n"

@@ -67,9 +67,20 @@ class Abi:
         self.lib = _lib.load()
         self.to_code = to_core_dtype
         self.dev = torch.device("cuda", 0)
+        # True: calls that name no options ask for the radix path where the library would pick
+        # the four-launch path for medium rows (tests of the radix kernels on small arrays)
+        self.force_radix = False
+        # default of local_sort's early_last_bytes (None: the library's own limit)
+        self.early_last_bytes = None
 
-    def describe_plan(self, dtype, volume, sort_dim_size, argsort):
-        return self._lib.describe_plan(self.to_code(np.dtype(dtype)), volume, sort_dim_size, argsort)
+    def describe_plan(self, dtype, volume, sort_dim_size, argsort, options=None):
+        if options is None and (self.force_radix or self.early_last_bytes is not None):
+            from cunumeric_amd._lib import Options
+
+            options = Options(early_last_min_bytes=-1 if self.early_last_bytes is None else self.early_last_bytes,
+                              bucket_path=0 if self.force_radix else -1)
+        return self._lib.describe_plan(self.to_code(np.dtype(dtype)), volume, sort_dim_size, argsort,
+                                       options=options)
 
     def _up(self, a):
         t = self.torch
@@ -79,9 +90,19 @@ class Abi:
         return t.from_numpy(a.reshape(-1).view(np.uint8).copy()).to(self.dev)
 
     def local_sort(self, values, sort_dim_size, argsort, indices_in=None, inplace=False,
-                   index_offset=0, want_values=False, chunks=0, static=False):
+                   index_offset=0, want_values=False, chunks=0, static=False, options=None,
+                   early_last_bytes=None):
         """chunks != 0: misort_local_chunked with that chunk target; static: misort_local_static
-        (the library's own scratch)."""
+        (the library's own scratch); options: a cunumeric_amd._lib.Options for misort_local_opts;
+        early_last_bytes: that field of the options alone."""
+        if early_last_bytes is None:
+            early_last_bytes = self.early_last_bytes
+        if options is None and not static and (early_last_bytes is not None or self.force_radix):
+            from cunumeric_amd._lib import Options
+
+            options = Options(target_chunks=chunks,
+                              early_last_min_bytes=-1 if early_last_bytes is None else early_last_bytes,
+                              bucket_path=0 if self.force_radix else -1)
         t = self.torch
         values = np.ascontiguousarray(values).reshape(-1)
         dt = values.dtype
@@ -105,6 +126,15 @@ class Abi:
         if static:
             rc = self.lib.misort_local_static(code, ptr(d_in), ptr(d_vout), ptr(d_iin), ptr(d_iout),
                                               volume, sort_dim_size, 1, index_offset, stream)
+        elif options is not None:
+            import ctypes
+
+            need = self.lib.misort_scratch_bytes_opts(code, volume, sort_dim_size, int(argsort),
+                                                      int(indices_in is not None), ctypes.byref(options))
+            scratch = t.empty(max(need, 256), dtype=t.uint8, device=self.dev)
+            rc = self.lib.misort_local_opts(code, ptr(d_in), ptr(d_vout), ptr(d_iin), ptr(d_iout),
+                                            volume, sort_dim_size, 1, index_offset,
+                                            scratch.data_ptr(), need, stream, ctypes.byref(options))
         elif chunks:
             need = self.lib.misort_scratch_bytes_chunked(code, volume, sort_dim_size, int(argsort),
                                                          int(indices_in is not None), chunks)
