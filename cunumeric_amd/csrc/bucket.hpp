@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "lanes.hpp"
+#include "radix.hpp"
 
 namespace misort {
 
@@ -52,13 +53,13 @@ struct BucketParams {
   uint32_t* bin_start;   // [BK_BINS + 1] first position of every bin, written by chunk 0 of the scatter
   uint32_t n;            // elements in the row
   uint32_t n_split;      // splitters in use
+  uint32_t oversample;   // samples per bin (BK_OVERSAMPLE at most)
   uint32_t tile, tiles_per_chunk, n_chunks, chunks_per_slab, n_slabs;
   uint32_t cap;          // longest bin sorted in registers
   int64_t index_offset;
   int xform;             // of the elements in keys_in
   int keys_travel;       // 1: the scatter writes keys (complex), 0: the elements themselves
   int rank_by_add;
-  int dbg_max_bits;
   int direct_equal;      // 1: the scatter writes the bins of equal keys straight to the outputs
                          // (outputs do not alias the inputs); 0: the bin sort copies them
 };
@@ -139,58 +140,62 @@ template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT>
 struct BlockSortSmem {
   uint32_t whist[(NT / 64) * RADIX];
   uint32_t wave_tot[NT / 64];
+  unsigned long long vary;
   __attribute__((aligned(16))) KeyT keys[NT * IPT];
   __attribute__((aligned(16))) PayT pay[HAS_PAY ? NT * IPT : 1];
 };
 
 struct BlockSortGeom {
-  uint32_t rows;   // rows of 64 elements in use
-  uint32_t R;      // rows per wavefront
+  uint32_t R;      // rows per wavefront: a power of two
   uint32_t wbase;  // element of this thread's slot 0
 };
 template <int NT>
 __device__ __forceinline__ BlockSortGeom block_sort_geom(uint32_t len)
 {
   BlockSortGeom g;
-  g.rows  = (len + 63) / 64;
-  g.R     = (g.rows + NT / 64 - 1) / (NT / 64);
-  g.wbase = (threadIdx.x >> 6) * g.R * 64 + (threadIdx.x & 63);
+  const uint32_t rows = (len + 63) / 64;
+  const uint32_t r    = (rows + NT / 64 - 1) / (NT / 64);
+  g.R                 = r <= 1 ? 1u : 1u << (32 - __builtin_clz(r - 1));
+  g.R                 = (uint32_t)__builtin_amdgcn_readfirstlane((int)g.R);
+  g.wbase             = (threadIdx.x >> 6) * g.R * 64 + (threadIdx.x & 63);
   return g;
 }
 
-template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT>
-__device__ __forceinline__ void block_radix_sort(uint32_t* whist /* (NT / 64) * RADIX */,
-                                                 uint32_t* wave_tot /* NT / 64 */,
-                                                 KeyT* skeys /* NT * IPT */, PayT* spay /* NT * IPT */,
-                                                 KeyT (&el)[IPT], PayT (&pay)[HAS_PAY ? IPT : 1],
-                                                 uint32_t len, KeyT base, int nbits, int xform, int by_add)
+// the passes for R = RR rows per wavefront: straight-line code over the RR slots (rows that
+// lie beyond the elements have no valid lane and do nothing)
+template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT, int RR>
+__device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t* wave_tot, KeyT* skeys,
+                                                      PayT* spay, KeyT (&el)[IPT],
+                                                      PayT (&pay)[HAS_PAY ? IPT : 1], uint32_t len, KeyT base,
+                                                      int nbits, int xform, int by_add, unsigned long long vary)
 {
-  static_assert(NT % RADIX == 0, "whole groups of one thread per digit value");
+  static_assert(NT % RADIX == 0 && RR <= IPT, "whole groups of one thread per digit value");
   constexpr int NW  = NT / 64;
   constexpr int NG  = NT / RADIX;  // thread groups, each covering all digit values
   constexpr int WPG = NW / NG;     // wavefronts whose counters a group rewrites
-  const int tid          = threadIdx.x;
-  const int lane         = tid & 63;
-  const int wave         = tid >> 6;
-  const BlockSortGeom g  = block_sort_geom<NT>(len);
-  const uint32_t R       = g.R;
-  const uint32_t wbase   = g.wbase;
-  uint32_t* my_hist      = whist + wave * RADIX;
-  const uint32_t dv      = tid & (RADIX - 1);
-  const int grp          = wave / (RADIX / 64);
+  const int tid        = threadIdx.x;
+  const int lane       = tid & 63;
+  const int wave       = tid >> 6;
+  const uint32_t wbase = (uint32_t)wave * (RR * 64) + lane;
+  uint32_t* my_hist    = whist + wave * RADIX;
+  const uint32_t dv    = tid & (RADIX - 1);
+  const int grp        = wave / (RADIX / 64);
+  const bool is_float  = xform == XF_FLOAT;
+  const KeyT flip      = xform == XF_SIGNED ? (KeyT)((KeyT)1 << (sizeof(KeyT) * 8 - 1)) : (KeyT)0;
   for (int shift = 0; shift < nbits; shift += RADIX_BITS) {
+    if (((vary >> shift) & (RADIX - 1)) == 0) continue;  // (same in every thread)
     for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
-    __syncthreads();
-    uint32_t d[IPT], r[IPT];
+    uint32_t d[RR], r[RR];
+    if (is_float) {
 #pragma unroll
-    for (int i = 0; i < IPT; ++i) {
-      if ((uint32_t)i < R && (uint32_t)wave * R + i < g.rows) {
-        const bool valid = wbase + i * 64 < len;
-        const KeyT k     = valid ? (KeyT)(KeyOps<KeyT>::to_key(el[i], xform) - base) : KeyOps<KeyT>::max_key();
-        d[i]             = KeyOps<KeyT>::digit(k, shift);
-        r[i]             = wave_rank<RADIX_BITS>(my_hist, d[i], valid, by_add);
-      }
+      for (int i = 0; i < RR; ++i) d[i] = KeyOps<KeyT>::digit((KeyT)(float_to_key(el[i]) - base), shift);
+    } else {
+#pragma unroll
+      for (int i = 0; i < RR; ++i) d[i] = KeyOps<KeyT>::digit((KeyT)((KeyT)(el[i] ^ flip) - base), shift);
     }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < RR; ++i) r[i] = wave_rank<RADIX_BITS>(my_hist, d[i], wbase + i * 64 < len, by_add);
     __syncthreads();
     // every thread takes digit value dv and the wavefronts of its group; all groups add up the
     // value's count over every wavefront and scan the counts over the digit values for themselves
@@ -215,23 +220,48 @@ __device__ __forceinline__ void block_radix_sort(uint32_t* whist /* (NT / 64) * 
       }
     }
     __syncthreads();
+    uint32_t q[RR];
 #pragma unroll
-    for (int i = 0; i < IPT; ++i) {
-      if ((uint32_t)i < R && wbase + i * 64 < len) {
-        const uint32_t q = my_hist[d[i]] + r[i];
-        skeys[q]         = el[i];
-        if constexpr (HAS_PAY) spay[q] = pay[i];
+    for (int i = 0; i < RR; ++i) q[i] = my_hist[d[i]] + r[i];
+#pragma unroll
+    for (int i = 0; i < RR; ++i) {
+      if (wbase + i * 64 < len) {
+        skeys[q[i]] = el[i];
+        if constexpr (HAS_PAY) spay[q[i]] = pay[i];
       }
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < IPT; ++i) {
-      if ((uint32_t)i < R && wbase + i * 64 < len) {
+    for (int i = 0; i < RR; ++i) {
+      if (wbase + i * 64 < len) {
         el[i] = skeys[wbase + i * 64];
         if constexpr (HAS_PAY) pay[i] = spay[wbase + i * 64];
       }
     }
   }
+}
+
+// xform: XF_UNSIGNED, XF_SIGNED or XF_FLOAT (complex keys are transformed before they get here)
+template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT>
+__device__ __forceinline__ void block_radix_sort(uint32_t* whist /* (NT / 64) * RADIX */,
+                                                 uint32_t* wave_tot /* NT / 64 */,
+                                                 KeyT* skeys /* NT * IPT */, PayT* spay /* NT * IPT */,
+                                                 KeyT (&el)[IPT], PayT (&pay)[HAS_PAY ? IPT : 1],
+                                                 uint32_t len, KeyT base, int nbits, int xform, int by_add,
+                                                 unsigned long long vary = ~0ull /* bits in which keys differ */)
+{
+  const uint32_t R = block_sort_geom<NT>(len).R;
+#define MISORT_BK_ROWS(RR)                                                                                   \
+  block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, IPT, RR>(whist, wave_tot, skeys, spay, el, pay, len, base, \
+                                                          nbits, xform, by_add, vary)
+  if (R == 1) MISORT_BK_ROWS(1);
+  else if (R == 2) MISORT_BK_ROWS(2);
+  else if (R == 4) MISORT_BK_ROWS(4);
+  else if constexpr (IPT >= 8) {
+    if (R == 8) MISORT_BK_ROWS(8);
+    else if constexpr (IPT >= 16) MISORT_BK_ROWS(16);
+  }
+#undef MISORT_BK_ROWS
 }
 
 // ---------------------------------------------------------------------------------------
@@ -246,7 +276,7 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
   for (uint32_t i = tid; i < p.n_slabs * BK_BINS; i += NT) p.slab_tot[i] = 0;
   // sample e of S comes from its own stretch of n / S elements, at a place inside it that a hash
   // of e picks (evenly spaced places would meet periodic data at the same phase every time)
-  const uint32_t S     = (p.n_split + 1) * BK_OVERSAMPLE;  // <= NT * IPT
+  const uint32_t S     = (p.n_split + 1) * p.oversample;  // <= NT * IPT
   const uint32_t span  = p.n / S > 0 ? p.n / S : 1;
   const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
   const BlockSortGeom g = block_sort_geom<NT>(S);
@@ -263,12 +293,36 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
     if (pos >= p.n) pos = p.n - 1;
     k[i] = ((uint32_t)i < g.R && e < S) ? KeyOps<KeyT>::to_key(in[pos], p.xform) : KeyOps<KeyT>::max_key();
   }
+  // which bits vary over the sample: passes over a digit that is the same in every sample key
+  // move nothing and are left out (the upper bytes of small integers, the low bytes of
+  // floats that hold integers)
+  {
+    __shared__ unsigned long long ref;
+    if (tid == 0) {
+      ref     = (unsigned long long)k[0];  // sample 0
+      sm.vary = 0;
+    }
+    __syncthreads();
+    const KeyT kr         = (KeyT)ref;
+    unsigned long long vv = 0;
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      if ((uint32_t)i < g.R && g.wbase + i * 64 < S) {
+        vv |= (unsigned long long)(KeyT)(k[i] ^ kr);
+        sm.keys[g.wbase + i * 64] = k[i];  // (if no pass runs at all, the sample is sorted as it is)
+      }
+    }
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) vv |= __shfl_xor(vv, sft, 64);
+    if ((tid & 63) == 0 && vv) atomicOr(&sm.vary, vv);
+    __syncthreads();
+  }
   block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
-                                                   (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add);
-  // the sorted sample is still in sm.keys; splitter t = sample 16 (t + 1) - 1
+                                                   (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, sm.vary);
+  // the sorted sample is still in sm.keys; splitter t = the last sample of stretch t
   KeyT* spl = reinterpret_cast<KeyT*>(p.splitters);
   for (uint32_t t = tid; t < BK_SLOTS; t += NT)
-    spl[t] = t < p.n_split ? sm.keys[(t + 1) * BK_OVERSAMPLE - 1] : KeyOps<KeyT>::max_key();
+    spl[t] = t < p.n_split ? sm.keys[(t + 1) * p.oversample - 1] : KeyOps<KeyT>::max_key();
 }
 
 // ---------------------------------------------------------------------------------------
@@ -289,19 +343,36 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
   const uint64_t b1    = b0 + clen < p.n ? b0 + clen : p.n;
   const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
   uint32_t* my         = hist + wave * BK_BINS;
-  // (four independent loads, then four searches side by side)
-  for (uint64_t i0 = b0; i0 < b1; i0 += 4 * NT) {
-    KeyT raw[4];
+  // (rounds of U independent loads per thread; the next round is asked for before this one is
+  // searched, U searches side by side)
+  constexpr int U = 4;
+  auto fetch = [&](KeyT (&raw)[U], uint64_t i0) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       const uint64_t i = i0 + (uint64_t)u * NT + tid;
       raw[u]           = in[i < b1 ? i : b0];
     }
+  };
+  auto consume = [&](const KeyT (&raw)[U], uint64_t i0) {
+    uint32_t b[U];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const uint64_t i = i0 + (uint64_t)u * NT + tid;
-      const uint32_t b = bin_of(tab, KeyOps<KeyT>::to_key(raw[u], p.xform));
-      if (i < b1) atomicAdd(&my[b], 1u);
+    for (int u = 0; u < U; ++u) b[u] = bin_of(tab, KeyOps<KeyT>::to_key(raw[u], p.xform));
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (i0 + (uint64_t)u * NT + tid < b1) atomicAdd(&my[b[u]], 1u);
+  };
+  {
+    KeyT ra[U], rb[U];
+    uint64_t i0 = b0;
+    if (i0 < b1) fetch(ra, i0);
+    while (i0 < b1) {
+      const uint64_t i1 = i0 + (uint64_t)U * NT, i2 = i1 + (uint64_t)U * NT;
+      if (i1 < b1) fetch(rb, i1);
+      consume(ra, i0);
+      if (i1 >= b1) break;
+      if (i2 < b1) fetch(ra, i2);
+      consume(rb, i1);
+      i0 = i2;
     }
   }
   __syncthreads();
@@ -338,6 +409,27 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t wbase = (uint32_t)wave * (64 * IPT) + lane;
   const uint32_t chunk = blockIdx.x;
+  const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
+  const uint32_t tile0 = chunk * p.tiles_per_chunk;
+  const uint32_t tiles = (p.n + TILE - 1) / TILE;
+  uint32_t tile_end    = tile0 + p.tiles_per_chunk;
+  if (tile_end > tiles) tile_end = tiles;
+  // the first tile is asked for before anything else: the splitters and the counts of the
+  // chunks before this one arrive meanwhile
+  KeyT el[IPT];
+  PayT pv[HAS_PAY ? IPT : 1];
+  auto load_tile = [&](uint32_t t) {
+    const uint32_t t0    = t * TILE;
+    const uint32_t valid = p.n - t0 < (uint32_t)TILE ? p.n - t0 : (uint32_t)TILE;
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) {
+      const uint32_t e = wbase + i * 64;
+      el[i]            = in[t0 + (e < valid ? e : 0u)];
+      if constexpr (PAY == PAY_I64) pv[i] = reinterpret_cast<const int64_t*>(p.pay_in)[t0 + (e < valid ? e : 0u)];
+      if constexpr (PAY == PAY_IDX32) pv[i] = t0 + e;
+    }
+  };
+  if (tile0 < tile_end) load_tile(tile0);
   load_splitters<KeyT, NT>(tab, reinterpret_cast<const KeyT*>(p.splitters));
 
   // ---- where this chunk's elements of every bin start: the bins before (all chunks), the
@@ -368,42 +460,28 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     __syncthreads();
   }
 
-  const KeyT* in   = reinterpret_cast<const KeyT*>(p.keys_in);
   KeyT* kbuf       = reinterpret_cast<KeyT*>(p.buf_keys[0]);
   PayT* pbuf       = reinterpret_cast<PayT*>(p.buf_pay[0]);
   KeyT* kout       = reinterpret_cast<KeyT*>(p.keys_out);
   int64_t* pout    = reinterpret_cast<int64_t*>(p.pay_out);
   uint32_t* my_hist = whist + wave * BK_BINS;
-  const uint32_t tile0 = chunk * p.tiles_per_chunk;
-  const uint32_t tiles = (p.n + TILE - 1) / TILE;
-  uint32_t tile_end    = tile0 + p.tiles_per_chunk;
-  if (tile_end > tiles) tile_end = tiles;
 
   for (uint32_t t = tile0; t < tile_end; ++t) {
     const uint32_t t0    = t * TILE;
     const uint32_t valid = p.n - t0 < (uint32_t)TILE ? p.n - t0 : (uint32_t)TILE;
-    KeyT el[IPT];
-    PayT pv[HAS_PAY ? IPT : 1];
     uint32_t b[IPT], r[IPT];
-#pragma unroll
-    for (int i = 0; i < IPT; ++i) {
-      const uint32_t e = wbase + i * 64;
-      el[i]            = in[t0 + (e < valid ? e : 0u)];
-      if constexpr (PAY == PAY_I64) pv[i] = reinterpret_cast<const int64_t*>(p.pay_in)[t0 + (e < valid ? e : 0u)];
-      if constexpr (PAY == PAY_IDX32) pv[i] = t0 + e;
-    }
     for (int i = tid; i < NW * BK_BINS; i += NT) whist[i] = 0;
-    __syncthreads();
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
-      const uint32_t e = wbase + i * 64;
-      const KeyT k     = KeyOps<KeyT>::to_key(el[i], p.xform);
+      const KeyT k = KeyOps<KeyT>::to_key(el[i], p.xform);
       if (p.keys_travel) el[i] = k;
-      // (slots past the end of the row in the last tile hold no key)
-      b[i] = e < valid ? bin_of(tab, k) : (uint32_t)(BK_BINS - 1);
-      r[i] = wave_rank<9>(my_hist, b[i], e < valid, p.rank_by_add);
+      b[i] = bin_of(tab, k);
     }
-    __syncthreads();
+    lds_barrier();
+    // (slots past the end of the row in the last tile hold no key)
+#pragma unroll
+    for (int i = 0; i < IPT; ++i) r[i] = wave_rank<9>(my_hist, b[i], wbase + i * 64 < valid, p.rank_by_add);
+    lds_barrier();
     uint32_t tot = 0;
     if (tid < BK_BINS) {
 #pragma unroll
@@ -411,7 +489,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     }
     const uint32_t incl = wave_incl_scan_u32(tot);
     if (tid < BK_BINS && lane == 63) wave_tot[wave] = incl;
-    __syncthreads();
+    lds_barrier();
     if (tid < BK_BINS) {
       uint32_t run = incl - tot;
       for (int w = 0; w < wave; ++w) run += wave_tot[w];
@@ -423,7 +501,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
         run += c;
       }
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
       if (wbase + i * 64 < valid) {
@@ -433,7 +511,9 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
         sbin[q] = (uint16_t)b[i];
       }
     }
-    __syncthreads();
+    // the next tile is asked for while this one is written out
+    if (t + 1 < tile_end) load_tile(t + 1);
+    lds_barrier();
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
       const uint32_t q = (uint32_t)tid + i * NT;
@@ -450,7 +530,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
     if (tid < BK_BINS) gpos[tid] += tot;
     // (the next tile's first barrier comes before anything reads gpos again)
   }
@@ -459,83 +539,159 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
 // ---------------------------------------------------------------------------------------
 // bin sort
 // ---------------------------------------------------------------------------------------
-// A bin too long for the registers: plain LSD passes by this one workgroup between the two
-// scratch buffers, NT elements at a time.  Splitters from a sorted sample leave this to inputs
-// built against the sampling; it is here so that those are sorted too.
-template <typename KeyT, int PAY>
-__device__ void bucket_sort_long(const BucketParams& p, uint32_t start, uint32_t len, KeyT base, int nbits,
-                                 int xform, uint32_t* whist /* (NT / 64) * RADIX */,
-                                 uint32_t* gbase /* RADIX */, uint32_t* wave_tot /* RADIX / 64 */)
+// A bin too long for the registers: LSD passes by this one workgroup between the two scratch
+// buffers, a tile of NT * IPT elements at a time.  Per pass one read of the bin counts the
+// digit, then the tiles are walked in order: rank within the tile, stage in LDS in
+// tile-sorted order, write every digit value's run to its place.  A bin that came out longer
+// than the sample promised is sorted this way (at about a third of the speed per element: the
+// runs are written in pieces of lines), and so is every bin of a row that a caller sends down
+// this path although it is longer than the path is meant for.
+template <typename KeyT, int PAY, int IPT>
+__device__ __forceinline__ void bucket_sort_long(
+  const BucketParams& p, uint32_t start, uint32_t len, KeyT base, int nbits, int xform, uint32_t* whist,
+  uint32_t* wave_tot, KeyT* skeys,
+  typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type* spay, uint32_t* gbase /* RADIX */,
+  uint32_t* tbase /* RADIX */)
 {
-  constexpr int NT = BK_NT, NW = NT / 64;
+  constexpr int NT = BK_NT, NW = NT / 64, TILE = NT * IPT;
+  constexpr int NG = NT / RADIX, WPG = NW / NG;
   using PayT = typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type;
+  constexpr bool HAS_PAY = PAY != PAY_NONE;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  uint32_t* my_hist = whist + wave * RADIX;
-  KeyT* kout        = reinterpret_cast<KeyT*>(p.keys_out);
-  int64_t* pout     = reinterpret_cast<int64_t*>(p.pay_out);
-  int cur           = 0;
-  for (int shift = 0; shift < nbits; shift += RADIX_BITS) {
-    const bool last  = shift + RADIX_BITS >= nbits;
+  const uint32_t wbase = (uint32_t)wave * (64 * IPT) + lane;
+  uint32_t* my_hist    = whist + wave * RADIX;
+  const uint32_t dv    = tid & (RADIX - 1);
+  const int grp        = wave / (RADIX / 64);
+  KeyT* kout           = reinterpret_cast<KeyT*>(p.keys_out);
+  int64_t* pout        = reinterpret_cast<int64_t*>(p.pay_out);
+  const bool is_float  = xform == XF_FLOAT;
+  const KeyT flip      = xform == XF_SIGNED ? (KeyT)((KeyT)1 << (sizeof(KeyT) * 8 - 1)) : (KeyT)0;
+  auto key_of = [&](KeyT raw) { return (KeyT)((is_float ? float_to_key(raw) : (KeyT)(raw ^ flip)) - base); };
+  const int npass = (nbits + RADIX_BITS - 1) / RADIX_BITS;  // <= 8
+
+  int cur = 0;
+  for (int ps = 0; ps < npass; ++ps) {
+    const int shift  = ps * RADIX_BITS;
+    const bool last  = ps == npass - 1;
     const KeyT* ksrc = reinterpret_cast<const KeyT*>(p.buf_keys[cur]) + start;
     const PayT* psrc = reinterpret_cast<const PayT*>(p.buf_pay[cur]) + start;
     KeyT* kdst       = reinterpret_cast<KeyT*>(p.buf_keys[cur ^ 1]) + start;
     PayT* pdst       = reinterpret_cast<PayT*>(p.buf_pay[cur ^ 1]) + start;
-    // counts of this digit over the bin, then where every digit value starts
-    for (int i = tid; i < RADIX; i += NT) gbase[i] = 0;
+    // ---- where every digit value starts in the bin: one read of the bin counts this pass's
+    // digit, every wavefront in counters of its own (atomics of several wavefronts on the same
+    // few words wait for one another), eight loads per thread in flight ----
+    for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
     __syncthreads();
-    for (uint32_t e = tid; e < len; e += NT)
-      atomicAdd(&gbase[KeyOps<KeyT>::digit((KeyT)(KeyOps<KeyT>::to_key(ksrc[e], xform) - base), shift)], 1u);
+    for (uint32_t e0 = 0; e0 < len; e0 += 8 * NT) {
+      KeyT raw[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const uint32_t e = e0 + u * NT + tid;
+        raw[u]           = ksrc[e < len ? e : 0u];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (e0 + u * NT + tid < len) atomicAdd(&my_hist[KeyOps<KeyT>::digit(key_of(raw[u]), shift)], 1u);
+    }
     __syncthreads();
     {
-      const uint32_t c    = tid < RADIX ? gbase[tid] : 0u;
+      uint32_t c = 0;
+      if (tid < RADIX) {
+#pragma unroll
+        for (int w = 0; w < NW; ++w) c += whist[w * RADIX + tid];
+      }
       const uint32_t incl = wave_incl_scan_u32(c);
       if (tid < RADIX && lane == 63) wave_tot[wave] = incl;
       __syncthreads();
       if (tid < RADIX) {
-        uint32_t s = incl - c;
-        for (int w = 0; w < wave; ++w) s += wave_tot[w];
-        gbase[tid] = s;
+        uint32_t s0 = incl - c;
+        for (int w = 0; w < wave; ++w) s0 += wave_tot[w];
+        gbase[tid] = s0;
       }
       __syncthreads();
     }
-    for (uint32_t t0 = 0; t0 < len; t0 += NT) {
-      const uint32_t e = t0 + tid;
-      const bool valid = e < len;
-      const KeyT el    = ksrc[valid ? e : 0u];
-      PayT pv{};
-      if constexpr (PAY != PAY_NONE) pv = psrc[valid ? e : 0u];
-      const uint32_t d = valid ? KeyOps<KeyT>::digit((KeyT)(KeyOps<KeyT>::to_key(el, xform) - base), shift) : 0u;
-      for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
-      __syncthreads();
-      const uint32_t r = wave_rank<RADIX_BITS>(my_hist, d, valid, p.rank_by_add);
-      __syncthreads();
-      uint32_t tot = 0;
-      if (tid < RADIX) {
+    KeyT el[IPT];
+    PayT pv[HAS_PAY ? IPT : 1];
+    auto load_tile = [&](uint32_t t0) {
+      const uint32_t valid = len - t0 < (uint32_t)TILE ? len - t0 : (uint32_t)TILE;
 #pragma unroll
-        for (int w = 0; w < NW; ++w) {
-          const uint32_t c       = whist[w * RADIX + tid];
-          whist[w * RADIX + tid] = tot;
-          tot += c;
+      for (int i = 0; i < IPT; ++i) {
+        const uint32_t e = wbase + i * 64;
+        el[i]            = ksrc[t0 + (e < valid ? e : 0u)];
+        if constexpr (HAS_PAY) pv[i] = psrc[t0 + (e < valid ? e : 0u)];
+      }
+    };
+    load_tile(0);
+    for (uint32_t t0 = 0; t0 < len; t0 += TILE) {
+      const uint32_t valid = len - t0 < (uint32_t)TILE ? len - t0 : (uint32_t)TILE;
+      for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
+      uint32_t d[IPT], r[IPT];
+#pragma unroll
+      for (int i = 0; i < IPT; ++i) d[i] = KeyOps<KeyT>::digit(key_of(el[i]), shift);
+      lds_barrier();
+#pragma unroll
+      for (int i = 0; i < IPT; ++i) r[i] = wave_rank<RADIX_BITS>(my_hist, d[i], wbase + i * 64 < valid, p.rank_by_add);
+      lds_barrier();
+      uint32_t count = 0, before = 0;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        if (w == grp * WPG) before = count;
+        count += whist[w * RADIX + dv];
+      }
+      const uint32_t incl = wave_incl_scan_u32(count);
+      if (lane == 63) wave_tot[wave] = incl;
+      lds_barrier();
+      {
+        uint32_t first = incl - count;
+        for (int w = grp * (RADIX / 64); w < wave; ++w) first += wave_tot[w];
+        if (grp == 0) tbase[dv] = first;
+        uint32_t off   = first + before;
+        uint32_t* mine = whist + grp * WPG * RADIX + dv;
+#pragma unroll
+        for (int w = 0; w < WPG; ++w) {
+          const uint32_t c = mine[w * RADIX];
+          mine[w * RADIX]  = off;
+          off += c;
         }
       }
-      __syncthreads();
-      if (valid) {
-        const uint32_t dst = gbase[d] + my_hist[d] + r;
-        if (last) {
-          if (kout) kout[start + dst] = el;
-          if constexpr (PAY == PAY_IDX32) pout[start + dst] = (int64_t)pv + p.index_offset;
-          if constexpr (PAY == PAY_I64) pout[start + dst] = pv;
-        } else {
-          kdst[dst] = el;
-          if constexpr (PAY != PAY_NONE) pdst[dst] = pv;
+      lds_barrier();
+#pragma unroll
+      for (int i = 0; i < IPT; ++i) {
+        if (wbase + i * 64 < valid) {
+          const uint32_t q = my_hist[d[i]] + r[i];
+          skeys[q]         = el[i];
+          if constexpr (HAS_PAY) spay[q] = pv[i];
         }
       }
-      __syncthreads();
-      if (tid < RADIX) gbase[tid] += tot;
-      __syncthreads();
+      // the next tile is asked for while this one is written out
+      if (t0 + TILE < len) load_tile(t0 + TILE);
+      lds_barrier();
+#pragma unroll
+      for (int i = 0; i < IPT; ++i) {
+        const uint32_t q = (uint32_t)tid + i * NT;
+        if (q < valid) {
+          const KeyT raw     = skeys[q];
+          const uint32_t dd  = KeyOps<KeyT>::digit(key_of(raw), shift);
+          const uint32_t dst = gbase[dd] + (q - tbase[dd]);
+          PayT pw{};
+          if constexpr (HAS_PAY) pw = spay[q];
+          if (last) {
+            if (kout) kout[start + dst] = raw;
+            if constexpr (PAY == PAY_IDX32) pout[start + dst] = (int64_t)pw + p.index_offset;
+            if constexpr (PAY == PAY_I64) pout[start + dst] = pw;
+          } else {
+            kdst[dst] = raw;
+            if constexpr (HAS_PAY) pdst[dst] = pw;
+          }
+        }
+      }
+      lds_barrier();
+      if (grp == 0) gbase[dv] += count;
+      // (three barriers of the next tile come before anything reads gbase or tbase again)
     }
-    // what this pass wrote to global memory is read by other threads of the workgroup next
-    __threadfence();
+    // What this pass wrote to global memory is read by other threads of this workgroup next:
+    // the barrier orders that at workgroup scope (the wavefronts of a workgroup share their
+    // CU's vector cache, which the stores went through).
     __syncthreads();
     cur ^= 1;
   }
@@ -552,6 +708,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   constexpr bool HAS_PAY = PAY != PAY_NONE;
   __shared__ BlockSortSmem<KeyT, PayT, HAS_PAY, NT, IPT> sm;
   __shared__ uint32_t gbase[RADIX];
+  __shared__ uint32_t tbase[RADIX];
   const int tid = threadIdx.x;
   const uint32_t g     = blockIdx.x;
   const uint32_t start = p.bin_start[2 * g], mid = p.bin_start[2 * g + 1], end = p.bin_start[2 * g + 2];
@@ -575,11 +732,11 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   const KeyT lo   = g > 0 ? spl[g - 1] : (KeyT)0;
   const KeyT hi   = spl[g];
   const unsigned long long diff = (unsigned long long)(KeyT)(hi - lo);
-  int nbits = diff ? 64 - __builtin_clzll(diff) : 0;
-  if (p.dbg_max_bits >= 0 && nbits > p.dbg_max_bits) nbits = p.dbg_max_bits;
+  const int nbits = diff ? 64 - __builtin_clzll(diff) : 0;
   const int xform = p.keys_travel ? (int)XF_UNSIGNED : p.xform;
   if (len > p.cap) {
-    bucket_sort_long<KeyT, PAY>(p, start, len, lo, nbits > 0 ? nbits : 1, xform, sm.whist, gbase, sm.wave_tot);
+    bucket_sort_long<KeyT, PAY, (IPT < 8 ? IPT : 8)>(p, start, len, lo, nbits > 0 ? nbits : 1, xform, sm.whist, sm.wave_tot, sm.keys,
+                                     sm.pay, gbase, tbase);
     return;
   }
   const BlockSortGeom geo = block_sort_geom<NT>(len);

@@ -338,7 +338,14 @@ struct Plan {
 // Slots per thread of the bin sort (1024 threads): the bin and its payload are staged in LDS
 // between the passes, 128 KB of it.
 constexpr int bucket_sort_ipt(int kb, int pay) { return kb + pay_bytes_of(pay) <= 8 ? 16 : 8; }
-constexpr int kBucketScatterIpt = 4;  // the scatter walks tiles of 4096 elements
+// The scatter walks tiles of 1024 * 4 elements while that gives every CU a chunk of at most two
+// tiles, and tiles as large as the staging area in LDS allows (element, payload, 2 bytes for the
+// bin) beyond that.
+constexpr int kBucketScatterIptSmall = 4;
+constexpr int bucket_scatter_ipt_large(int kb, int pay)
+{
+  return kb + pay_bytes_of(pay) <= 4 ? 16 : (kb + pay_bytes_of(pay) <= 8 ? 8 : 4);
+}
 
 // Number of chunks a row-set is cut into.  Two per CU measured best from 2^24 to 2^28 keys:
 // long chunks keep the downsweep's pipeline and its carried partial lines busy (with one
@@ -415,7 +422,10 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // a bin four times the average does not happen), and there are at most 256 of them.
     const size_t cap = opt.bucket_cap ? std::min<size_t>(opt.bucket_cap, (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay))
                                       : (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay);
-    const size_t max_len = opt.bucket_path > 0 ? (size_t)0xFFFFFFFFu / 2 : 64 * cap;
+    // (up to 256 bins of half of what the registers hold on average: with 16 samples per bin a
+    // bin twice the average is a one-in-a-thousand event, and such a bin is still sorted, by
+    // the slower loop through global memory)
+    const size_t max_len = opt.bucket_path > 0 ? (size_t)0xFFFFFFFFu / 2 : 128 * cap;
     if (pl.row_len <= max_len && cap >= 64) {
       size_t bins = opt.bucket_bins ? opt.bucket_bins : (pl.row_len + 1023) / 1024;
       if (bins < 2) bins = 2;
@@ -434,7 +444,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
   };
 
   if (pl.strategy == S_BUCKET) {
-    pl.bk_tile            = BK_NT * kBucketScatterIpt;
+    pl.bk_tile            = BK_NT * (pl.row_len <= ((size_t)1 << 21) ? kBucketScatterIptSmall
+                                                                       : bucket_scatter_ipt_large(pl.dt.bytes, pl.pay));
     const size_t tiles    = (pl.row_len + pl.bk_tile - 1) / pl.bk_tile;
     const size_t want     = tiles < 256 ? tiles : 256;
     pl.bk_tiles_per_chunk = (uint32_t)((tiles + want - 1) / want);
@@ -867,6 +878,7 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a)
   p.bin_start       = reinterpret_cast<uint32_t*>(S + pl.off_bk_bin_start);
   p.n               = (uint32_t)pl.row_len;
   p.n_split         = pl.bk_split;
+  p.oversample      = BK_OVERSAMPLE;
   p.tile            = pl.bk_tile;
   p.tiles_per_chunk = pl.bk_tiles_per_chunk;
   p.n_chunks        = pl.bk_chunks;
@@ -877,7 +889,6 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a)
   p.xform           = pl.dt.xform;
   p.keys_travel     = pl.dt.xform == XF_COMPLEX ? 1 : 0;
   p.rank_by_add     = rank_by_add_on_current_device();
-  p.dbg_max_bits    = getenv("DBG_MAX_BITS") ? atoi(getenv("DBG_MAX_BITS")) : -1;
   p.direct_equal    = (a.values_out == nullptr || a.values_out != a.values_in) &&
                       (a.indices_out == nullptr || a.indices_out != a.indices_in);
   constexpr int IPT = bucket_sort_ipt(sizeof(KeyT), PAY);
@@ -888,8 +899,12 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a)
     hipLaunchKernelGGL((bucket_count_kernel<KeyT>), dim3(pl.bk_chunks), dim3(BK_COUNT_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_SCATTER, [&] {
-    hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, kBucketScatterIpt>), dim3(pl.bk_chunks), dim3(BK_NT), 0,
-                       L.stream, p);
+    constexpr int LARGE = bucket_scatter_ipt_large(sizeof(KeyT), PAY);
+    if (pl.bk_tile == (uint32_t)BK_NT * kBucketScatterIptSmall)
+      hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, kBucketScatterIptSmall>), dim3(pl.bk_chunks),
+                         dim3(BK_NT), 0, L.stream, p);
+    else
+      hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, LARGE>), dim3(pl.bk_chunks), dim3(BK_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_SORT, [&] {
     hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(pl.bk_split + 1), dim3(BK_NT), 0, L.stream, p);

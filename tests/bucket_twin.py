@@ -32,8 +32,8 @@ def bin_of(sorted_spl: np.ndarray, tree: np.ndarray, keys: np.ndarray) -> np.nda
     return 2 * j + (sorted_spl[j] == keys)
 
 
-def sample_places(n: int, n_split: int) -> np.ndarray:
-    s = (n_split + 1) * OVERSAMPLE
+def sample_places(n: int, n_split: int, oversample: int = OVERSAMPLE) -> np.ndarray:
+    s = (n_split + 1) * oversample
     e = np.arange(s, dtype=np.uint64)
     h = (e * np.uint64(0x9E3779B1)) & np.uint64(0xFFFFFFFF)
     h ^= h >> np.uint64(15)

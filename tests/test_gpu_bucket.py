@@ -135,12 +135,24 @@ def test_bins_too_long_for_the_registers(abi, dtype):
     assert np.array_equal(got, pay[np.argsort(a, kind="stable")])
 
 
-def test_rows_beyond_the_built_in_limit_when_asked_for(abi):
+@pytest.mark.parametrize("dtype", [np.int16, np.int32, np.float32, np.int64, np.float64, np.complex64],
+                         ids=lambda d: np.dtype(d).name)
+def test_rows_of_several_million_elements_when_asked_for(abi, dtype):
+    """Rows beyond what 256 bins of register size hold do not take this path by themselves;
+    asked for, every bin is a few tiles long and is sorted tile by tile through global memory,
+    and the scatter walks its largest tiles, several per chunk."""
     rng = np.random.default_rng(76)
-    n = (1 << 21) + 5
-    for dtype in (np.int32, np.float64):
-        a = random_array(dtype, n, rng)
-        check(abi, a, options=Options(bucket_path=1))
+    o = Options(bucket_path=1)
+    for n in ((1 << 21) + 5, (1 << 22) + 4099):
+        for narrow in (False, True):
+            a = random_array(dtype, n, rng, narrow=narrow)
+            print(f"bucket dtype={np.dtype(dtype).name} n={n} narrow={narrow} "
+                  f"plan={abi.describe_plan(dtype, n, n, True, options=o)}", flush=True)
+            assert "strategy=bucket" in abi.describe_plan(dtype, n, n, True, options=o)
+            check(abi, a, options=o)
+    pay = rng.integers(-2**62, 2**62, n, dtype=np.int64)
+    got = abi.local_sort(a, n, argsort=True, indices_in=pay, inplace=True, options=o)
+    assert np.array_equal(got, pay[np.argsort(a, kind="stable")])
 
 
 def test_path_can_be_switched_off_per_call(abi):
