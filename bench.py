@@ -113,12 +113,36 @@ def cpu_model() -> str:
     return "unknown CPU"
 
 
+def cpu_physical_cores() -> int:
+    """Distinct (package, core) pairs among the CPUs this process may run on."""
+    try:
+        allowed = os.sched_getaffinity(0)
+        cores, cur = set(), {}
+        with open("/proc/cpuinfo") as f:
+            for line in f.read().split("\n") + [""]:
+                if ":" in line:
+                    k, v = [x.strip() for x in line.split(":", 1)]
+                    cur[k] = v
+                elif cur:
+                    if int(cur.get("processor", -1)) in allowed:
+                        cores.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+                    cur = {}
+        return len(cores) or len(allowed)
+    except (OSError, ValueError, AttributeError):
+        return os.cpu_count() or 1
+
+
 def cpu_baseline(sample: np.ndarray, code: int, row: int, argsort: bool, threads: int) -> dict:
     """The reference's CPU/OpenMP variant (oracle/cpu_variant.cc: Thrust stable sort per row
     under omp::par, as in sort_cpu.inl:40-69) timed on `threads` host cores: median of three
     runs of std::chrono-equivalent wall time around the sort call only."""
     path = os.path.join(ROOT, "oracle", "libcpu_variant.so")
-    host = f"{cpu_model()}, {os.cpu_count()} logical CPUs on the host, {threads} threads used"
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    host = (f"{cpu_model()}; {os.cpu_count()} logical CPUs on the host, {usable} usable by this process on "
+            f"{cpu_physical_cores()} physical cores; {threads} OpenMP threads used")
     if not os.path.exists(path):
         return {"value": None, "unit": "Gkeys/s", "cores": threads, "kind": "port", "host": host,
                 "sample": "oracle/libcpu_variant.so not built"}
@@ -787,6 +811,13 @@ def main() -> int:
             elif name in ("count16_hist", "count16_fill"):
                 # counting sort of 2-byte values: one read for the counts, one write
                 b, dominant = k_bytes, "count16_hist"
+            elif name.startswith("bucket_") and name != "bucket_plan":
+                # medium rows: count reads the elements; scatter reads them and writes them with
+                # 32-bit positions; the bin sort reads those and writes the result
+                vp = 4 if argsort else 0
+                b = {"bucket_count": k_bytes, "bucket_scatter": 2 * k_bytes + vp,
+                     "bucket_sort": k_bytes + vp + (v_bytes if argsort else k_bytes)}[name]
+                dominant = "bucket_sort"
             else:
                 continue
             l = kk["launches_per_step"]
@@ -799,12 +830,38 @@ def main() -> int:
             per_pass[name] = {"bytes_per_key": b, "GB/s": gbs, "frac": gbs / HBM_PEAK_GBS}
         achieved = tot_bytes / (tot_ms * 1e-3) / 1e9 if tot_ms else 0.0
         n_up = kernels.get("upsweep", {}).get("launches_per_step", 0)
-        if "upsweep" in kernels:
-            gbs = k_bytes * n / (kernels["upsweep"]["avg_ms"] * 1e-3) / 1e9
-            per_pass["upsweep"] = {"bytes_per_key": k_bytes, "GB/s": gbs, "frac": gbs / HBM_PEAK_GBS}
+        if "upsweep" in kernels and n_up:
+            # The first upsweep reads the keys.  A later one reads either the keys again or, where
+            # the pass before left the digit side-band, one byte per key (plan side_band=1: every
+            # later upsweep; side_band=2: decided per row on the device).  Each launch is priced
+            # by what it read: with side_band=2 a launch that would exceed the device's pure read
+            # rate (7 TB/s) at key width must have read bytes.
+            side = 1 if "side_band=1" in plan else (2 if "side_band=2" in plan else 0)
+            ups = medians["upsweep"]
+            ran_up = ups >= 0.05 * ups.max()
+            keys_ms, byte_ms = [], []
+            for i, (ms_i, r_i) in enumerate(zip(ups, ran_up)):
+                if not r_i:
+                    continue
+                bytes_read = i > 0 and (side == 1 or (side == 2 and k_bytes * n / (ms_i * 1e-3) / 1e9 > 7000.0))
+                (byte_ms if bytes_read else keys_ms).append(float(ms_i))
+            if keys_ms:
+                gbs = k_bytes * n / (np.mean(keys_ms) * 1e-3) / 1e9
+                per_pass["upsweep"] = {"bytes_per_key": k_bytes, "launches": len(keys_ms), "GB/s": gbs,
+                                       "frac": gbs / HBM_PEAK_GBS}
+            if byte_ms:
+                gbs = n / (np.mean(byte_ms) * 1e-3) / 1e9
+                per_pass["upsweep_side_band"] = {"bytes_per_key": 1, "launches": len(byte_ms), "GB/s": gbs,
+                                                 "frac": gbs / HBM_PEAK_GBS}
         # whole sort: one histogram read + the passes (an LSD sort's minimum with a single
         # up-front histogram; this implementation reads the keys once more per pass)
         b_total = tot_bytes / n + (k_bytes if n_up else 0)
+        if "strategy=bucket" in plan:
+            # priced like the radix sort it stands in for (8-bit digits over the whole key: one
+            # histogram read, P passes), so that the fraction compares with the radix path's
+            P = k_bytes
+            b_total = (k_bytes + 2 * k_bytes * P) if not argsort else \
+                (4 * k_bytes + 3 * v_bytes + (P - 2) * (2 * k_bytes + 2 * v_bytes))
         traffic = None
         if args.workload == "c2" and log2n == 28:
             # from the rocprofv3 --pmc runs summarised in
@@ -829,6 +886,12 @@ def main() -> int:
             "algorithmic_bytes_per_launch": tot_bytes / max(n_launch, 1),
             "avg_launch_ms": tot_ms / max(n_launch, 1),
             "per_pass": per_pass,
+            # the pass furthest from the roofline, and how many scatter passes ran (planned
+            # passes whose digit no key varies in return at once and are not counted)
+            "per_pass_min": (min(per_pass.items(), key=lambda kv: kv[1]["frac"])[0] if per_pass else None),
+            "per_pass_min_frac": (min(v["frac"] for v in per_pass.values()) if per_pass else None),
+            "passes_executed": sum(kk["launches_per_step"] for name, kk in kernels.items()
+                                   if name.startswith("downsweep_")),
             # whole call: algorithmic bytes of all passes + one histogram read, over the time
             # of one call from its first launch to its last kernel's end (HIP events)
             "whole_sort": {"bytes_per_key": b_total, "call_ms": call_ms, "kernel_ms_sum": all_ms,

@@ -61,3 +61,29 @@ def test_static_scratch_refuses_what_does_not_fit():
     assert bool((d_out == 0x5A).all())  # nothing was launched
     # empty input: nothing to do
     assert abi.lib.misort_local_static(code, None, None, None, None, 0, 0, 1, 0, None) == 0
+
+
+def test_static_scratch_call_allocates_nothing():
+    """With inputs and outputs in place before the call, the call itself leaves the device's
+    free memory and torch's own allocator untouched (the first call of the process on this GPU
+    has looked the buffer's address up and probed the LDS already: misort_init)."""
+    abi = Abi()
+    t = abi.torch
+    assert abi.lib.misort_init() == 0
+    rng = np.random.default_rng(78)
+    n = 400_003
+    a = random_array(np.float32, n, rng)
+    code = abi.to_code(a.dtype)
+    d_in = t.from_numpy(a.view(np.uint8).copy()).to(abi.dev)
+    d_out = t.empty(n * 8, dtype=t.uint8, device=abi.dev)
+    st = t.cuda.current_stream().cuda_stream
+    t.cuda.synchronize()
+    free0, _ = t.cuda.mem_get_info()
+    alloc0, reserved0 = t.cuda.memory_allocated(), t.cuda.memory_reserved()
+    for _ in range(3):
+        assert abi.lib.misort_local_static(code, d_in.data_ptr(), None, None, d_out.data_ptr(), n, n, 1, 0, st) == 0
+    t.cuda.synchronize()
+    free1, _ = t.cuda.mem_get_info()
+    assert (t.cuda.memory_allocated(), t.cuda.memory_reserved()) == (alloc0, reserved0)
+    assert free1 == free0
+    assert np.array_equal(d_out.cpu().numpy().view(np.int64), np.argsort(a, kind="stable"))
