@@ -774,10 +774,21 @@ def main() -> int:
         medians = {name: np.median(np.asarray(v, dtype=np.float64).reshape(reps, -1), axis=0)
                    for name, v in acc.items()}
         longest_scatter = max([m.max() for name, m in medians.items() if name.startswith("downsweep_")] or [0.0])
+        # Long rows try the four-launch path first (plan low_cardinality_attempt): either its
+        # count / scatter / bin sort kernels return at once (many distinct keys) or, if it went
+        # through, every kernel of the radix path does.
+        bucket_ms = medians["bucket_scatter"].max() if "bucket_scatter" in medians else 0.0
+        attempt = "low_cardinality_attempt" in plan
+        bucket_done = attempt and bucket_ms > 20 * longest_scatter
+        bucket_dead = attempt and not bucket_done
         for name, v in acc.items():
             per_call = np.asarray(v, dtype=np.float64).reshape(reps, -1)
             per_launch = medians[name]
-            if name == "upsweep":
+            if bucket_done and (name == "upsweep" or name.startswith("downsweep_")):
+                ran = np.zeros_like(per_launch, dtype=bool)
+            elif bucket_dead and name in ("bucket_count", "bucket_scatter", "bucket_sort"):
+                ran = np.zeros_like(per_launch, dtype=bool)
+            elif name == "upsweep":
                 ran = per_launch >= 0.05 * per_launch.max()
             elif name in ("downsweep_middle", "downsweep_last"):
                 ran = per_launch >= 0.05 * longest_scatter
@@ -815,9 +826,16 @@ def main() -> int:
                 # medium rows: count reads the elements; scatter reads them and writes them with
                 # 32-bit positions; the bin sort reads those and writes the result
                 vp = 4 if argsort else 0
-                b = {"bucket_count": k_bytes, "bucket_scatter": 2 * k_bytes + vp,
-                     "bucket_sort": k_bytes + vp + (v_bytes if argsort else k_bytes)}[name]
-                dominant = "bucket_sort"
+                if "strategy=bucket" in plan:
+                    b = {"bucket_count": k_bytes, "bucket_scatter": 2 * k_bytes + vp,
+                         "bucket_sort": k_bytes + vp + (v_bytes if argsort else k_bytes)}[name]
+                    dominant = "bucket_sort"
+                elif name == "bucket_sort":
+                    continue  # (few distinct keys: nothing is left for the bin sort)
+                else:
+                    # few distinct keys: the scatter reads the elements and writes the result
+                    b = {"bucket_count": k_bytes, "bucket_scatter": k_bytes + (v_bytes if argsort else k_bytes)}[name]
+                    dominant = "bucket_scatter"
             else:
                 continue
             l = kk["launches_per_step"]
@@ -856,7 +874,7 @@ def main() -> int:
         # whole sort: one histogram read + the passes (an LSD sort's minimum with a single
         # up-front histogram; this implementation reads the keys once more per pass)
         b_total = tot_bytes / n + (k_bytes if n_up else 0)
-        if "strategy=bucket" in plan:
+        if "strategy=bucket" in plan or bucket_done:
             # priced like the radix sort it stands in for (8-bit digits over the whole key: one
             # histogram read, P passes), so that the fraction compares with the radix path's
             P = k_bytes

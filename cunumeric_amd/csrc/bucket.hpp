@@ -62,6 +62,16 @@ struct BucketParams {
   int rank_by_add;
   int direct_equal;      // 1: the scatter writes the bins of equal keys straight to the outputs
                          // (outputs do not alias the inputs); 0: the bin sort copies them
+  // Long rows, which the radix path serves: this path is tried first where the keys take few
+  // distinct values (every value a bin of its own, filled by the scatter; nothing left to
+  // sort), and the radix kernels that follow return at once if it went through.
+  //   flags[0]  set by the plan kernel: go on (the sample holds at most 255 distinct keys, which
+  //             then are the splitters; or attempt == 2, which tries with any sample)
+  //   flags[1]  set by the scatter: done (no bin that needs sorting is longer than cap);
+  //             the bin sort runs if it is set, the radix kernels if it is not
+  // NULL: the path runs unconditionally.
+  uint32_t* flags;
+  int attempt;           // 0: not an attempt; 1: only with few distinct sample keys; 2: always
 };
 
 // Rank of this lane's key among the keys with the same digit value that the wavefront has
@@ -321,6 +331,42 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
                                                    (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, sm.vary);
   // the sorted sample is still in sm.keys; splitter t = the last sample of stretch t
   KeyT* spl = reinterpret_cast<KeyT*>(p.splitters);
+  if (p.attempt) {
+    // an attempt on a long row: if the sample holds at most 255 distinct keys, those are the
+    // splitters, each with a bin of equal keys behind it
+    __shared__ uint32_t wave_heads[NT / 64];
+    const int lane = tid & 63, wave = tid >> 6;
+    constexpr int PER = IPT;  // sample keys [PER * tid, PER * tid + PER) per thread
+    uint32_t heads = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const uint32_t e = (uint32_t)tid * PER + j;
+      heads += (e < S && (e == 0 || sm.keys[e] != sm.keys[e - 1])) ? 1u : 0u;
+    }
+    const uint32_t incl = wave_incl_scan_u32(heads);
+    if (lane == 63) wave_heads[wave] = incl;
+    __syncthreads();
+    uint32_t first = incl - heads, total = 0;
+    for (int w = 0; w < NT / 64; ++w) {
+      if (w < wave) first += wave_heads[w];
+      total += wave_heads[w];
+    }
+    const bool few = total <= (uint32_t)(BK_SLOTS - 1);
+    if (few) {
+      for (uint32_t t = tid; t < BK_SLOTS; t += NT) spl[t] = KeyOps<KeyT>::max_key();
+      __syncthreads();  // (the padding is in place before the distinct keys go over it)
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const uint32_t e = (uint32_t)tid * PER + j;
+        if (e < S && (e == 0 || sm.keys[e] != sm.keys[e - 1])) spl[first++] = sm.keys[e];
+      }
+    }
+    if (tid == 0) {
+      p.flags[0] = (few || p.attempt == 2) ? 1u : 0u;
+      p.flags[1] = 0u;
+    }
+    if (few) return;
+  }
   for (uint32_t t = tid; t < BK_SLOTS; t += NT)
     spl[t] = t < p.n_split ? sm.keys[(t + 1) * p.oversample - 1] : KeyOps<KeyT>::max_key();
 }
@@ -334,6 +380,7 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
   constexpr int NT = BK_COUNT_NT, NW = NT / 64;
   __shared__ SplitterTable<KeyT> tab;
   __shared__ uint32_t hist[NW * BK_BINS];
+  if (p.flags && p.flags[0] == 0) return;  // an attempt that the plan kernel called off
   const int tid = threadIdx.x, wave = tid >> 6;
   for (int i = tid; i < NW * BK_BINS; i += NT) hist[i] = 0;
   load_splitters<KeyT, NT>(tab, reinterpret_cast<const KeyT*>(p.splitters));
@@ -406,6 +453,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
   __shared__ __attribute__((aligned(16))) PayT spay[HAS_PAY ? TILE : 1];
   __shared__ uint16_t sbin[TILE];
 
+  if (p.flags && p.flags[0] == 0) return;  // an attempt that the plan kernel called off
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t wbase = (uint32_t)wave * (64 * IPT) + lane;
   const uint32_t chunk = blockIdx.x;
@@ -447,7 +495,23 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     }
     const uint32_t incl = wave_incl_scan_u32(tot);
     if (tid < BK_BINS && lane == 63) wave_tot[wave] = incl;
+    if (p.flags) {
+      // an attempt goes through only if every bin that needs sorting fits the registers of the
+      // bin sort: decided from the bins' totals, the same way by every workgroup
+      uint32_t longest = (tid < BK_BINS && (tid & 1) == 0) ? tot : 0u;
+#pragma unroll
+      for (int sft = 32; sft > 0; sft >>= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, sft, 64));
+      if (tid < BK_BINS && lane == 0) bin_base[wave] = longest;  // (bin_base is free until the first tile)
+    }
     __syncthreads();
+    if (p.flags) {
+      uint32_t longest = 0;
+      for (int w = 0; w < BK_BINS / 64; ++w) longest = max(longest, bin_base[w]);
+      const bool ok = longest <= p.cap;
+      if (chunk == 0 && tid == 0) p.flags[1] = ok ? 1u : 0u;
+      if (!ok) return;
+      __syncthreads();
+    }
     if (tid < BK_BINS) {
       uint32_t start = incl - tot;
       for (int w = 0; w < wave; ++w) start += wave_tot[w];
@@ -709,6 +773,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   __shared__ BlockSortSmem<KeyT, PayT, HAS_PAY, NT, IPT> sm;
   __shared__ uint32_t gbase[RADIX];
   __shared__ uint32_t tbase[RADIX];
+  if (p.flags && p.flags[1] == 0) return;  // an attempt that did not go through
   const int tid = threadIdx.x;
   const uint32_t g     = blockIdx.x;
   const uint32_t start = p.bin_start[2 * g], mid = p.bin_start[2 * g + 1], end = p.bin_start[2 * g + 2];

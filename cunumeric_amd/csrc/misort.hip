@@ -138,6 +138,8 @@ struct PlanOptions {
   int bucket_path = -1;                 // < 0: the built-in choice; 0: never; > 0: wherever it is able to run
   unsigned bucket_bins = 0;             // 0: the built-in choice; else splitter intervals, 2 .. 256
   unsigned bucket_cap = 0;              // 0: the built-in choice; else the longest bin sorted in registers
+  int low_cardinality = -1;             // long rows try the four-launch path first: < 0: where the sample holds
+                                        // few distinct keys; 0: never; 2: with any sample
 };
 
 static int fail(int code, const std::string& msg)
@@ -332,6 +334,10 @@ struct Plan {
   // sample -> count -> scatter -> sort the bins (bucket.hpp): geometry and scratch
   uint32_t bk_split = 0, bk_cap = 0, bk_tile = 0, bk_tiles_per_chunk = 0, bk_chunks = 0, bk_slabs = 0;
   size_t off_bk_splitters = 0, off_bk_slab_tot = 0, off_bk_chunk_hist = 0, off_bk_bin_start = 0;
+  // radix plans of one long row: the four-launch path is tried first, and goes through where
+  // the keys take few distinct values (1: if the sample says so; 2: tried with any sample)
+  int low_card = 0;
+  size_t off_bk_flags = 0;
   size_t total = 0;
 };
 
@@ -344,7 +350,7 @@ constexpr int bucket_sort_ipt(int kb, int pay) { return kb + pay_bytes_of(pay) <
 constexpr int kBucketScatterIptSmall = 4;
 constexpr int bucket_scatter_ipt_large(int kb, int pay)
 {
-  return kb + pay_bytes_of(pay) <= 4 ? 16 : (kb + pay_bytes_of(pay) <= 8 ? 8 : 4);
+  return kb + pay_bytes_of(pay) <= 4 ? 16 : (kb + pay_bytes_of(pay) <= 12 ? 8 : 4);
 }
 
 // Number of chunks a row-set is cut into.  Two per CU measured best from 2^24 to 2^28 keys:
@@ -443,7 +449,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     return o;
   };
 
-  if (pl.strategy == S_BUCKET) {
+  // chunks of the count and scatter kernels of the four-launch path, and its tables
+  auto bucket_tables = [&] {
     pl.bk_tile            = BK_NT * (pl.row_len <= ((size_t)1 << 21) ? kBucketScatterIptSmall
                                                                        : bucket_scatter_ipt_large(pl.dt.bytes, pl.pay));
     const size_t tiles    = (pl.row_len + pl.bk_tile - 1) / pl.bk_tile;
@@ -455,6 +462,11 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.off_bk_slab_tot    = take((size_t)pl.bk_slabs * BK_BINS * sizeof(uint32_t));
     pl.off_bk_chunk_hist  = take((size_t)pl.bk_chunks * BK_BINS * sizeof(uint32_t));
     pl.off_bk_bin_start   = take((BK_BINS + 1) * sizeof(uint32_t));
+    pl.off_bk_flags       = take(2 * sizeof(uint32_t));
+  };
+
+  if (pl.strategy == S_BUCKET) {
+    bucket_tables();
     for (int b = 0; b < 2; ++b) pl.off_keys[b] = take(pl.volume * pl.dt.bytes);
     if (pl.pay != PAY_NONE)
       for (int b = 0; b < 2; ++b) pl.off_pay[b] = take(pl.volume * (pl.pay == PAY_IDX32 ? 4 : 8));
@@ -534,6 +546,21 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     if (pl.gather_values) {
       pl.off_gather_idx = take(pl.volume * sizeof(int64_t));
       pl.off_gather_src = take(pl.volume * pl.dt.bytes);  // copy of the input when in == out
+    }
+    // One long row of 4- or 8-byte keys: the four-launch path is tried first (its plan kernel
+    // alone, 15 us, where the sample holds more than 255 distinct keys).  With few distinct
+    // values every one of them is a splitter with a bin of equal keys behind it, which the
+    // scatter fills in input order at the elements' final places: one read to count, one read
+    // and one write to place, against a read and a write per key byte.  It shares the radix
+    // path's two key and payload buffers.  (Not for keys-only float sorts, whose zeros and NaNs
+    // the radix path patches with kernels of its own, and not in place: the scatter writes
+    // results while other workgroups still read the input.)
+    if (opt.low_cardinality != 0 && pl.rows == 1 && (pl.dt.bytes == 4 || pl.dt.bytes == 8) && pl.n_passes >= 3 &&
+        !pl.gather_values && !pl.specials && pl.row_len < 0xFFFFFFFFull) {
+      pl.low_card = opt.low_cardinality == 2 ? 2 : 1;
+      pl.bk_split = BK_SLOTS - 1;
+      pl.bk_cap   = (uint32_t)(BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay));
+      bucket_tables();
     }
   } else if (pl.strategy == S_COUNT16) {
     // one histogram workgroup per CU and half of the key range, a few rounds of them
@@ -663,6 +690,9 @@ static void launch_zero(Launcher& L, void* p, size_t bytes)
 }
 
 template <typename KeyT, int PAY>
+static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int attempt = 0);
+
+template <typename KeyT, int PAY>
 static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
 {
   const size_t eb    = sizeof(KeyT);
@@ -687,6 +717,17 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   unsigned long long* special_blk =
     reinterpret_cast<unsigned long long*>(S + pl.off_special_blk);
 
+  // few distinct keys: the four-launch path writes the result, and the kernels below return at once
+  const uint32_t* done_flag = nullptr;
+  if constexpr (sizeof(KeyT) == 4 || sizeof(KeyT) == 8) {
+    const bool outputs_apart = (a.values_out == nullptr || a.values_out != a.values_in) &&
+                               (a.indices_out == nullptr || a.indices_out != a.indices_in);
+    if (pl.low_card && outputs_apart) {
+      bucket_sort_row<KeyT, PAY>(L, pl, a, pl.low_card);
+      done_flag = reinterpret_cast<const uint32_t*>(S + pl.off_bk_flags) + 1;
+    }
+  }
+
   launch_zero(L, S + pl.off_special_ctr, pl.zero_bytes);
 
   const size_t pay_bytes     = PAY == PAY_IDX32 ? 4 : 8;
@@ -710,6 +751,7 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
   pp.xform           = pl.dt.xform;
   pp.rank_by_add     = rank_by_add_on_current_device();
+  pp.done_flag       = done_flag;
   pp.n_rows          = (uint32_t)pl.rows;
   pp.key_buf[0]      = S + pl.off_keys[0];
   pp.key_buf[1]      = S + pl.off_keys[1];
@@ -860,10 +902,12 @@ static void radix_sort_dispatch(Launcher& L, const Plan& pl, const SortArgs& a)
 // one row through sample -> count -> scatter -> sort the bins (bucket.hpp)
 // ---------------------------------------------------------------------------------------
 template <typename KeyT, int PAY>
-static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a)
+static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int attempt)
 {
   char* S = a.scratch;
   BucketParams p{};
+  p.attempt         = attempt;
+  p.flags           = attempt ? reinterpret_cast<uint32_t*>(S + pl.off_bk_flags) : nullptr;
   p.keys_in         = a.values_in;
   p.pay_in          = a.indices_in;
   p.keys_out        = a.values_out;
@@ -907,7 +951,8 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a)
       hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, LARGE>), dim3(pl.bk_chunks), dim3(BK_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_SORT, [&] {
-    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(pl.bk_split + 1), dim3(BK_NT), 0, L.stream, p);
+    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(attempt ? BK_SLOTS : pl.bk_split + 1), dim3(BK_NT),
+                       0, L.stream, p);
   });
 }
 
@@ -1034,7 +1079,8 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   if (!dtype_info(dtype, dt)) return fail(MISORT_ERR_DTYPE, "unknown dtype code");
   // (the selection walks the chunks of the radix plan)
   PlanOptions radix_only;
-  radix_only.bucket_path = 0;
+  radix_only.bucket_path     = 0;
+  radix_only.low_cardinality = 0;
   int rc = make_plan(dtype, volume, sort_dim_size, want_indices, false, u.pl, radix_only);
   if (rc != MISORT_OK) return rc;
   // 1- and 2-byte values are counted, which beats selecting; their positions are selected
@@ -1412,6 +1458,7 @@ static PlanOptions plan_options(const misort_options* o)
     opt.bucket_path          = o->bucket_path;
     opt.bucket_bins          = o->bucket_bins;
     opt.bucket_cap           = o->bucket_cap;
+    opt.low_cardinality      = o->low_cardinality;
   }
   return opt;
 }
@@ -1517,6 +1564,10 @@ int misort_describe_plan_opts(int dtype, size_t volume, size_t sort_dim_size, in
     const size_t len = strlen(buf);
     if (len + 64 < buf_bytes)
       snprintf(buf + len, buf_bytes - len, " bins=%u bin_cap=%u chunks=%u", pl.bk_split + 1, pl.bk_cap, pl.bk_chunks);
+  }
+  if (pl.low_card) {
+    const size_t len = strlen(buf);
+    if (len + 32 < buf_bytes) snprintf(buf + len, buf_bytes - len, " low_cardinality_attempt=%d", pl.low_card);
   }
   if (pl.skip_dead_passes) {
     const size_t len = strlen(buf);

@@ -101,6 +101,10 @@ struct PassParams {
   int shift;
   int xform;
   int rank_by_add;    // downsweep: rank with returning LDS adds where the chunk's digits allow
+  // Non-NULL where the four-launch path (bucket.hpp) was tried on this row first: the word is 1
+  // if that path has written the result already, and every kernel of the radix path then
+  // returns at once.
+  const uint32_t* done_flag;
 };
 
 // key_bits holds this many copies of its four words (their OR counts)
@@ -289,6 +293,7 @@ template <int NT>
 __global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
 {
   __shared__ __attribute__((aligned(16))) uint32_t h[RADIX * 32];
+  if (p.done_flag && *p.done_flag) return;
   for (int i = threadIdx.x; i < RADIX * 32; i += NT) h[i] = 0;  // (while the plan's words arrive)
   const bool skip = plan_pass(p).skip;
   __syncthreads();
@@ -312,6 +317,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   constexpr int WORDS  = NW * RADIX * COPIES > RADIX * 32 ? NW * RADIX * COPIES : RADIX * 32;
   __shared__ __attribute__((aligned(16))) uint32_t lhist[WORDS];
   __shared__ unsigned long long wg_bits[FIRST ? NW * 4 : 1];
+  if (p.done_flag && *p.done_flag) return;
   const uint32_t row   = blockIdx.x / p.chunks_per_row;
   const uint32_t chunk = blockIdx.x % p.chunks_per_row;
   // (the counters are cleared while the words of the plan arrive)
@@ -616,6 +622,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   __shared__ unsigned long long b_pos[SIDE ? RADIX : 1];
   __shared__ uint32_t b_tab[SIDE ? RADIX : 1];
 
+  if (p.done_flag && *p.done_flag) return;
   const int tid        = threadIdx.x;
   const int lane       = tid & 63;
   const int wave       = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -247,8 +247,8 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
 
 /*
  * misort_scratch_bytes / misort_local with choices that are otherwise built in, per call (a
- * NULL pointer or a zeroed struct with early_last_min_bytes = bucket_path = -1 means "as
- * misort_local").  No counterpart in the reference; for tests that have to reach the code for
+ * NULL pointer, or a zeroed struct with early_last_min_bytes = bucket_path = low_cardinality
+ * = -1, means "as misort_local").  No counterpart in the reference; for tests that have to reach the code for
  * large or unusual inputs with small arrays, and for measurements.  Give the query and the
  * sort the same options.
  *   target_chunks         as misort_local_chunked (0: built in)
@@ -262,6 +262,13 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *   bucket_bins           number of bins, 2 .. 256 (0: built in, one per 1024 elements)
  *   bucket_cap            longest bin that is sorted in registers; longer ones take the
  *                         workgroup's loop through global memory (0: built in, 8192 or 16384)
+ *   low_cardinality       single rows too long for that path, 4- and 8-byte keys, outputs apart
+ *                         from the inputs: the path is tried all the same where a sample of the
+ *                         row holds at most 255 distinct keys (each of them then gets a bin of
+ *                         its own, which needs no sorting), and the radix kernels return at once
+ *                         if it went through; decided on the device, nothing is read back.
+ *                         < 0: built in (on); 0: never; 2: tried with any sample (tests of the
+ *                         way back to the radix path)
  */
 typedef struct misort_options {
   size_t target_chunks;
@@ -269,6 +276,7 @@ typedef struct misort_options {
   int bucket_path;
   unsigned bucket_bins;
   unsigned bucket_cap;
+  int low_cardinality;
 } misort_options;
 size_t misort_scratch_bytes_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                                  int has_indices_in, const misort_options* options);
