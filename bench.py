@@ -874,7 +874,7 @@ def main() -> int:
         # whole sort: one histogram read + the passes (an LSD sort's minimum with a single
         # up-front histogram; this implementation reads the keys once more per pass)
         b_total = tot_bytes / n + (k_bytes if n_up else 0)
-        if "strategy=bucket" in plan or bucket_done:
+        if "strategy=bucket" in plan:
             # priced like the radix sort it stands in for (8-bit digits over the whole key: one
             # histogram read, P passes), so that the fraction compares with the radix path's
             P = k_bytes
