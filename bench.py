@@ -587,6 +587,87 @@ def run_axis(args) -> int:
     return 0 if ok else 1
 
 
+def run_sizes(args) -> int:
+    """--workload sizes: single rows of 2^14 + 1 ... 2^21 elements (the sizes between the row
+    kernels and the long rows of the radix path), int32 / float32 / int64, sort and stable
+    argsort: one call timed alone with HIP events (median of 30) and back to back, the built-in
+    plan beside the radix path asked for through misort_local_opts.  Not the headline."""
+    import torch
+
+    from cunumeric_amd import _lib
+    from cunumeric_amd._lib import Options
+    from cunumeric_amd.config import to_core_dtype
+
+    lib = _lib.load()
+    dev = torch.device("cuda", 0)
+    _lib.check(lib.misort_init())
+    stream = torch.cuda.current_stream().cuda_stream
+    rows, ok_all = [], True
+
+    def one(dtype, n, argsort, opts):
+        rng = np.random.Generator(np.random.PCG64(1))
+        if np.dtype(dtype).kind in "iu":
+            ii = np.iinfo(dtype)
+            a = rng.integers(ii.min, ii.max, n, dtype=dtype, endpoint=True)
+        else:
+            a = rng.random(n).astype(dtype)
+        code = to_core_dtype(np.dtype(dtype))
+        d_in = torch.from_numpy(a.view(np.uint8)).to(dev)
+        d_out = torch.empty(n * 8, dtype=torch.uint8, device=dev)
+        need = lib.misort_scratch_bytes_opts(code, n, n, int(argsort), 0, ctypes.byref(opts))
+        scr = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        vo, io = (None, d_out.data_ptr()) if argsort else (d_out.data_ptr(), None)
+
+        def call():
+            _lib.check(lib.misort_local_opts(code, d_in.data_ptr(), vo, None, io, n, n, 1, 0, scr.data_ptr(),
+                                             need, stream, ctypes.byref(opts)))
+
+        for _ in range(5):
+            call()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(30):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            call()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3)
+        t0 = time.perf_counter()
+        for _ in range(30):
+            call()
+        torch.cuda.synchronize()
+        b2b = (time.perf_counter() - t0) / 30 * 1e6
+        if argsort:
+            ok = bool(np.array_equal(d_out.cpu().numpy().view(np.int64), np.argsort(a, kind="stable")))
+        else:
+            ok = d_out[: a.nbytes].cpu().numpy().tobytes() == np.sort(a, kind="stable").tobytes()
+        return float(np.median(ts)), b2b, ok
+
+    for dtype in (np.int32, np.float32, np.int64):
+        for argsort in (False, True):
+            for lg in range(14, 22):
+                n = (1 << lg) + (1 if lg == 14 else 0)
+                code = to_core_dtype(np.dtype(dtype))
+                plan = _lib.describe_plan(code, n, n, argsort).split()[0]
+                d = one(dtype, n, argsort, Options())
+                r = one(dtype, n, argsort, Options(bucket_path=0, low_cardinality=0))
+                ok_all = ok_all and d[2] and r[2]
+                rows.append({"dtype": np.dtype(dtype).name, "argsort": argsort, "log2n": lg, "plan": plan,
+                             "call_us": round(d[0], 1), "back_to_back_us": round(d[1], 1),
+                             "radix_call_us": round(r[0], 1), "radix_back_to_back_us": round(r[1], 1)})
+    out = {
+        "metric": "microseconds per call, single rows of 2^14 .. 2^21 elements, 1 MI355X",
+        "value": next(x["back_to_back_us"] for x in rows if x["dtype"] == "int32" and not x["argsort"] and x["log2n"] == 20),
+        "unit": "us (int32 sort of 2^20, back to back)", "n_gpus": 1, "steps": 30, "warmup": 5,
+        "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic", "config": {"workload": "sizes sweep: uniform int32 / float32 / int64, sort and stable argsort"},
+        "parity_guard": "ok" if ok_all else "FAILED", "sizes": rows,
+    }
+    print(json.dumps(out))
+    return 0 if ok_all else 1
+
+
 def gpu_library_baseline(workload: str, log2n: int):
     """The reference's device work for this workload (index fill + copy + CUB radix sort,
     src/cunumeric/sort/sort.cu:1694-1751 and cub_sort.cuh:36-189) served by hipCUB / rocPRIM on
@@ -613,7 +694,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ss", "uniq", "part", "sel", "axis"], default="c2")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ss", "uniq", "part", "sel", "axis", "sizes"], default="c2")
     ap.add_argument("--log2n", type=int, default=None)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true")
@@ -643,6 +724,8 @@ def main() -> int:
         return run_partition(args)
     if args.workload == "sel":
         return run_select(args)
+    if args.workload == "sizes":
+        return run_sizes(args)
     dev = torch.device("cuda", 0)
     title, gen, def_log2n, argsort, row = WORKLOADS[args.workload]
     log2n = args.log2n if args.log2n is not None else def_log2n

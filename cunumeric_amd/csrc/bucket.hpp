@@ -192,9 +192,9 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
   const int grp        = wave / (RADIX / 64);
   const bool is_float  = xform == XF_FLOAT;
   const KeyT flip      = xform == XF_SIGNED ? (KeyT)((KeyT)1 << (sizeof(KeyT) * 8 - 1)) : (KeyT)0;
+  for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;  // (a pass leaves them cleared for the next)
   for (int shift = 0; shift < nbits; shift += RADIX_BITS) {
     if (((vary >> shift) & (RADIX - 1)) == 0) continue;  // (same in every thread)
-    for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
     uint32_t d[RR], r[RR];
     if (is_float) {
 #pragma unroll
@@ -241,6 +241,7 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
       }
     }
     __syncthreads();
+    for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;  // (read for the last time before the barrier)
 #pragma unroll
     for (int i = 0; i < RR; ++i) {
       if (wbase + i * 64 < len) {

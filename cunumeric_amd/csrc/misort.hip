@@ -138,8 +138,10 @@ struct PlanOptions {
   int bucket_path = -1;                 // < 0: the built-in choice; 0: never; > 0: wherever it is able to run
   unsigned bucket_bins = 0;             // 0: the built-in choice; else splitter intervals, 2 .. 256
   unsigned bucket_cap = 0;              // 0: the built-in choice; else the longest bin sorted in registers
-  int low_cardinality = -1;             // long rows try the four-launch path first: < 0: where the sample holds
-                                        // few distinct keys; 0: never; 2: with any sample
+  unsigned bucket_oversample = 0;       // 0: the built-in choice; else samples per bin, 1 .. 16
+  int low_cardinality = -1;             // long rows try the four-launch path first: < 0: rows of 2^27 elements
+                                        // and more, where the sample holds few distinct keys; 0: never;
+                                        // 1: the same for every length; 2: with any sample
 };
 
 static int fail(int code, const std::string& msg)
@@ -333,6 +335,7 @@ struct Plan {
   size_t c16_chunks = 0, c16_chunk_len = 0, off_c16_hist = 0, off_c16_prefix = 0;
   // sample -> count -> scatter -> sort the bins (bucket.hpp): geometry and scratch
   uint32_t bk_split = 0, bk_cap = 0, bk_tile = 0, bk_tiles_per_chunk = 0, bk_chunks = 0, bk_slabs = 0;
+  uint32_t bk_oversample = BK_OVERSAMPLE;
   size_t off_bk_splitters = 0, off_bk_slab_tot = 0, off_bk_chunk_hist = 0, off_bk_bin_start = 0;
   // radix plans of one long row: the four-launch path is tried first, and goes through where
   // the keys take few distinct values (1: if the sample says so; 2: tried with any sample)
@@ -439,6 +442,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
       pl.strategy = S_BUCKET;
       pl.bk_split = (uint32_t)bins - 1;
       pl.bk_cap   = (uint32_t)cap;
+      if (opt.bucket_oversample >= 1 && opt.bucket_oversample <= (unsigned)BK_OVERSAMPLE)
+        pl.bk_oversample = opt.bucket_oversample;
     }
   }
 
@@ -555,8 +560,11 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // path's two key and payload buffers.  (Not for keys-only float sorts, whose zeros and NaNs
     // the radix path patches with kernels of its own, and not in place: the scatter writes
     // results while other workgroups still read the input.)
-    if (opt.low_cardinality != 0 && pl.rows == 1 && (pl.dt.bytes == 4 || pl.dt.bytes == 8) && pl.n_passes >= 3 &&
-        !pl.gather_values && !pl.specials && pl.row_len < 0xFFFFFFFFull) {
+    // (By itself from 2^27 elements on: the plan kernel and the three launches that return at
+    // once cost 35-50 us, which is 1 % of a sort of 2^28 keys and 14 % of one of 2^24.)
+    if (opt.low_cardinality != 0 && (opt.low_cardinality > 0 || pl.row_len >= ((size_t)1 << 27)) && pl.rows == 1 &&
+        (pl.dt.bytes == 4 || pl.dt.bytes == 8) && pl.n_passes >= 3 && !pl.gather_values && !pl.specials &&
+        pl.row_len < 0xFFFFFFFFull) {
       pl.low_card = opt.low_cardinality == 2 ? 2 : 1;
       pl.bk_split = BK_SLOTS - 1;
       pl.bk_cap   = (uint32_t)(BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay));
@@ -922,7 +930,7 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int 
   p.bin_start       = reinterpret_cast<uint32_t*>(S + pl.off_bk_bin_start);
   p.n               = (uint32_t)pl.row_len;
   p.n_split         = pl.bk_split;
-  p.oversample      = BK_OVERSAMPLE;
+  p.oversample      = pl.bk_oversample;
   p.tile            = pl.bk_tile;
   p.tiles_per_chunk = pl.bk_tiles_per_chunk;
   p.n_chunks        = pl.bk_chunks;
@@ -1459,6 +1467,7 @@ static PlanOptions plan_options(const misort_options* o)
     opt.bucket_bins          = o->bucket_bins;
     opt.bucket_cap           = o->bucket_cap;
     opt.low_cardinality      = o->low_cardinality;
+    opt.bucket_oversample    = o->bucket_oversample;
   }
   return opt;
 }

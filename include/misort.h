@@ -262,13 +262,16 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *   bucket_bins           number of bins, 2 .. 256 (0: built in, one per 1024 elements)
  *   bucket_cap            longest bin that is sorted in registers; longer ones take the
  *                         workgroup's loop through global memory (0: built in, 8192 or 16384)
+ *   bucket_oversample     sample keys drawn per bin, 1 .. 16 (0: built in, 16; fewer samples give
+ *                         uneven bins: tests of bins that outgrow the registers)
  *   low_cardinality       single rows too long for that path, 4- and 8-byte keys, outputs apart
  *                         from the inputs: the path is tried all the same where a sample of the
  *                         row holds at most 255 distinct keys (each of them then gets a bin of
  *                         its own, which needs no sorting), and the radix kernels return at once
  *                         if it went through; decided on the device, nothing is read back.
- *                         < 0: built in (on); 0: never; 2: tried with any sample (tests of the
- *                         way back to the radix path)
+ *                         < 0: built in (rows of 2^27 elements and more: the attempt costs
+ *                         35-50 us where it is called off); 0: never; 1: rows of any length;
+ *                         2: tried with any sample (tests of the way back to the radix path)
  */
 typedef struct misort_options {
   size_t target_chunks;
@@ -277,6 +280,7 @@ typedef struct misort_options {
   unsigned bucket_bins;
   unsigned bucket_cap;
   int low_cardinality;
+  unsigned bucket_oversample;
 } misort_options;
 size_t misort_scratch_bytes_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                                  int has_indices_in, const misort_options* options);

@@ -155,6 +155,18 @@ def test_rows_of_several_million_elements_when_asked_for(abi, dtype):
     assert np.array_equal(got, pay[np.argsort(a, kind="stable")])
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.float64], ids=lambda d: np.dtype(d).name)
+def test_uneven_bins_from_a_thin_sample(abi, dtype):
+    """One sample key per bin: bin lengths spread like an exponential distribution, so that at
+    a million elements a few bins outgrow the registers and take the loop through global
+    memory, next to bins of a handful of elements."""
+    rng = np.random.default_rng(78)
+    for n in (1 << 20, 700001):
+        a = random_array(dtype, n, rng)
+        check(abi, a, options=Options(bucket_oversample=1))
+        check(abi, a, options=Options(bucket_oversample=3, bucket_cap=2048))
+
+
 def test_path_can_be_switched_off_per_call(abi):
     rng = np.random.default_rng(77)
     a = random_array(np.float32, 50001, rng)

@@ -22,6 +22,9 @@ def abi():
     return Abi()
 
 
+ON = dict(options=Options(low_cardinality=1))  # (by itself the attempt is made from 2^27 elements on)
+
+
 def check(abi, a, **kw):
     n = a.size
     assert np.array_equal(abi.local_sort(a, n, argsort=True, **kw), np.argsort(a, kind="stable"))
@@ -48,10 +51,12 @@ def zipf_values(dtype, n, k, rng):
 def test_few_distinct_values(abi, dtype, k):
     rng = np.random.default_rng(81)
     a = zipf_values(dtype, N, k, rng)
-    plan = abi.describe_plan(dtype, N, N, True)
+    plan = abi.describe_plan(dtype, N, N, True, **ON)
     print(f"low cardinality dtype={np.dtype(dtype).name} k={k} plan={plan}", flush=True)
     assert "strategy=radix" in plan and "low_cardinality_attempt=1" in plan
-    check(abi, a)
+    assert "low_cardinality_attempt" not in abi.describe_plan(dtype, N, N, True)
+    assert "low_cardinality_attempt=1" in abi.describe_plan(dtype, 1 << 27, 1 << 27, True)
+    check(abi, a, **ON)
 
 
 @pytest.mark.parametrize("dtype", [np.int32, np.int64, np.float64], ids=lambda d: np.dtype(d).name)
@@ -62,11 +67,11 @@ def test_rare_values_between_the_common_ones(abi, dtype):
     a = zipf_values(dtype, N, 250, rng)
     rare = rng.random(N) < 0.01
     a[rare] = random_array(dtype, int(rare.sum()), rng, specials=False)
-    check(abi, a)
+    check(abi, a, **ON)
     pay = rng.integers(-2**62, 2**62, N, dtype=np.int64)
-    got = abi.local_sort(a, N, argsort=True, indices_in=pay)
+    got = abi.local_sort(a, N, argsort=True, indices_in=pay, **ON)
     assert np.array_equal(got, pay[np.argsort(a, kind="stable")])
-    got = abi.local_sort(a, N, argsort=True, index_offset=-77)
+    got = abi.local_sort(a, N, argsort=True, index_offset=-77, **ON)
     assert np.array_equal(got, np.argsort(a, kind="stable") - 77)
 
 
@@ -79,30 +84,31 @@ def test_way_back_to_the_radix_path(abi, dtype):
     rng = np.random.default_rng(83)
     a = random_array(dtype, N, rng)
     check(abi, a, options=Options(low_cardinality=2))
-    check(abi, a)  # built in: the plan kernel alone sees that the values are many
+    check(abi, a, **ON)  # the plan kernel alone sees that the values are many
     check(abi, a, options=Options(low_cardinality=0))
     b = zipf_values(dtype, N, 12, rng)
     b[rng.integers(0, N, N // 50)] = random_array(dtype, N // 50, rng, specials=False)[0]
     idx = rng.integers(0, N, 300000)
     b[idx] = random_array(dtype, idx.size, rng, specials=False)  # many rare values: bins too long
-    check(abi, b)
+    check(abi, b, **ON)
     check(abi, b, options=Options(low_cardinality=2))
 
 
 def test_in_place_keeps_the_radix_path(abi):
     rng = np.random.default_rng(84)
     a = zipf_values(np.int64, N, 16, rng)
-    assert bits_equal(abi.local_sort(a, N, argsort=False, inplace=True), np.sort(a, kind="stable"))
+    assert bits_equal(abi.local_sort(a, N, argsort=False, inplace=True, **ON), np.sort(a, kind="stable"))
     pay = rng.integers(-2**62, 2**62, N, dtype=np.int64)
-    got = abi.local_sort(a, N, argsort=True, indices_in=pay, inplace=True)
+    got = abi.local_sort(a, N, argsort=True, indices_in=pay, inplace=True, **ON)
     assert np.array_equal(got, pay[np.argsort(a, kind="stable")])
 
 
 def test_unique_and_python_surface(abi):
+    """2^27 elements: the built-in plan makes the attempt."""
     import cunumeric_amd as num
 
     rng = np.random.default_rng(85)
-    a = zipf_values(np.int64, N, 40, rng)
+    a = zipf_values(np.int32, 1 << 27, 40, rng)
     assert np.array_equal(np.asarray(num.unique(num.array(a))), np.unique(a))
     assert np.array_equal(np.asarray(num.argsort(num.array(a), kind="stable")), np.argsort(a, kind="stable"))
     assert np.array_equal(np.asarray(num.sort(num.array(a))), np.sort(a))
