@@ -87,3 +87,51 @@ def test_static_scratch_call_allocates_nothing():
     assert (t.cuda.memory_allocated(), t.cuda.memory_reserved()) == (alloc0, reserved0)
     assert free1 == free0
     assert np.array_equal(d_out.cpu().numpy().view(np.int64), np.argsort(a, kind="stable"))
+
+
+def test_static_scratch_call_recorded_into_a_graph():
+    """misort_init outside the capture, then misort_local_static recorded into a HIP graph
+    (its launches only: the call allocates nothing, synchronises nothing and clears its
+    counters with kernels, not memsets).  The graph is replayed with new inputs, eager work and
+    synchronisations in between, and every replay is checked against NumPy."""
+    abi = Abi()
+    t = abi.torch
+    assert abi.lib.misort_init() == 0
+    rng = np.random.default_rng(79)
+    for dtype, n, argsort in ((np.float32, 300_001, True), (np.int64, 1_200_000, False), (np.int32, 50_000, True)):
+        code = abi.to_code(np.dtype(dtype))
+        nbytes = n * np.dtype(dtype).itemsize
+        d_in = t.zeros(nbytes, dtype=t.uint8, device=abi.dev)
+        d_out = t.zeros(n * 8, dtype=t.uint8, device=abi.dev)
+        a0 = random_array(dtype, n, rng)
+        d_in.copy_(t.from_numpy(a0.view(np.uint8).copy()))
+        # one eager call first (whatever lazy set-up the runtime does for these kernels)
+        vo, io = (None, d_out.data_ptr()) if argsort else (d_out.data_ptr(), None)
+        st = t.cuda.current_stream().cuda_stream
+        assert abi.lib.misort_local_static(code, d_in.data_ptr(), vo, None, io, n, n, 1, 0, st) == 0
+        t.cuda.synchronize()
+        g = t.cuda.CUDAGraph()
+        side = t.cuda.Stream()
+        side.wait_stream(t.cuda.current_stream())
+        with t.cuda.stream(side):
+            g.capture_begin()
+            rc = abi.lib.misort_local_static(code, d_in.data_ptr(), vo, None, io, n, n, 1, 0, side.cuda_stream)
+            g.capture_end()
+        assert rc == 0, abi.lib.misort_last_error()
+        t.cuda.current_stream().wait_stream(side)
+        for rep in range(4):
+            a = random_array(dtype, n, rng, narrow=(rep == 2))
+            d_in.copy_(t.from_numpy(a.view(np.uint8).copy()))
+            d_out.zero_()
+            t.cuda.synchronize()
+            g.replay()
+            t.cuda.synchronize()
+            got = d_out.cpu().numpy()
+            if argsort:
+                assert np.array_equal(got.view(np.int64), np.argsort(a, kind="stable")), (dtype, rep)
+            else:
+                assert bits_equal(got[:nbytes].view(a.dtype), np.sort(a, kind="stable")), (dtype, rep)
+            # eager work between the replays
+            m = min(n, 70_001)
+            assert bits_equal(abi.local_sort(a[:m], m, argsort=False), np.sort(a[:m], kind="stable"))
+        del g
