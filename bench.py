@@ -604,7 +604,8 @@ def run_sizes(args) -> int:
     stream = torch.cuda.current_stream().cuda_stream
     rows, ok_all = [], True
 
-    def one(dtype, n, argsort, opts):
+    def one(dtype, n, argsort, opts, row_len=None):
+        row_len = row_len or n
         rng = np.random.Generator(np.random.PCG64(1))
         if np.dtype(dtype).kind in "iu":
             ii = np.iinfo(dtype)
@@ -614,12 +615,12 @@ def run_sizes(args) -> int:
         code = to_core_dtype(np.dtype(dtype))
         d_in = torch.from_numpy(a.view(np.uint8)).to(dev)
         d_out = torch.empty(n * 8, dtype=torch.uint8, device=dev)
-        need = lib.misort_scratch_bytes_opts(code, n, n, int(argsort), 0, ctypes.byref(opts))
+        need = lib.misort_scratch_bytes_opts(code, n, row_len, int(argsort), 0, ctypes.byref(opts))
         scr = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
         vo, io = (None, d_out.data_ptr()) if argsort else (d_out.data_ptr(), None)
 
         def call():
-            _lib.check(lib.misort_local_opts(code, d_in.data_ptr(), vo, None, io, n, n, 1, 0, scr.data_ptr(),
+            _lib.check(lib.misort_local_opts(code, d_in.data_ptr(), vo, None, io, n, row_len, 1, 0, scr.data_ptr(),
                                              need, stream, ctypes.byref(opts)))
 
         for _ in range(5):
@@ -638,10 +639,12 @@ def run_sizes(args) -> int:
             call()
         torch.cuda.synchronize()
         b2b = (time.perf_counter() - t0) / 30 * 1e6
+        a2 = a.reshape(-1, row_len)
         if argsort:
-            ok = bool(np.array_equal(d_out.cpu().numpy().view(np.int64), np.argsort(a, kind="stable")))
+            ok = bool(np.array_equal(d_out.cpu().numpy().view(np.int64).reshape(a2.shape),
+                                     np.argsort(a2, axis=1, kind="stable")))
         else:
-            ok = d_out[: a.nbytes].cpu().numpy().tobytes() == np.sort(a, kind="stable").tobytes()
+            ok = d_out[: a.nbytes].cpu().numpy().tobytes() == np.sort(a2, axis=1, kind="stable").tobytes()
         return float(np.median(ts)), b2b, ok
 
     for dtype in (np.int32, np.float32, np.int64):
@@ -654,6 +657,19 @@ def run_sizes(args) -> int:
                 r = one(dtype, n, argsort, Options(bucket_path=0, low_cardinality=0))
                 ok_all = ok_all and d[2] and r[2]
                 rows.append({"dtype": np.dtype(dtype).name, "argsort": argsort, "log2n": lg, "plan": plan,
+                             "call_us": round(d[0], 1), "back_to_back_us": round(d[1], 1),
+                             "radix_call_us": round(r[0], 1), "radix_back_to_back_us": round(r[1], 1)})
+    # several rows side by side (rows too long for the row kernels, 2^20 elements in all)
+    for dtype in (np.int32, np.int64):
+        for argsort in (False, True):
+            for n_rows in (2, 8, 32):
+                row_len = (1 << 20) // n_rows
+                code = to_core_dtype(np.dtype(dtype))
+                plan = _lib.describe_plan(code, 1 << 20, row_len, argsort).split()[0]
+                d = one(dtype, 1 << 20, argsort, Options(), row_len)
+                r = one(dtype, 1 << 20, argsort, Options(bucket_path=0, low_cardinality=0), row_len)
+                ok_all = ok_all and d[2] and r[2]
+                rows.append({"dtype": np.dtype(dtype).name, "argsort": argsort, "log2n": 20, "rows": n_rows, "plan": plan,
                              "call_us": round(d[0], 1), "back_to_back_us": round(d[1], 1),
                              "radix_call_us": round(r[0], 1), "radix_back_to_back_us": round(r[1], 1)})
     out = {

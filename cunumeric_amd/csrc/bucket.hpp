@@ -1,4 +1,4 @@
-// Sort of one row of a few ten thousand to about a million elements in four launches: sample
+// Sort of rows of a few ten thousand to about a million elements in four launches: sample
 // -> count -> scatter -> sort the bins.  It serves the sizes where the radix path's two
 // launches per digit are mostly launch and start-up time (the reference's own benchmark sorts
 // 10^6 elements, examples/sort.py:110-123; the calls replaced are the same ones,
@@ -51,7 +51,11 @@ struct BucketParams {
   uint32_t* chunk_hist;  // [n_chunks][BK_BINS]
   uint32_t* slab_tot;    // [n_slabs][BK_BINS], cleared by the plan kernel
   uint32_t* bin_start;   // [BK_BINS + 1] first position of every bin, written by chunk 0 of the scatter
-  uint32_t n;            // elements in the row
+  // Several rows of the same length are sorted side by side: the second launch dimension is the
+  // row, and every pointer above (but flags) is the first row's: row r has its elements at
+  // r * n, its splitters at r * BK_SLOTS, its slab totals at r * n_slabs * BK_BINS, its chunk
+  // counts at r * n_chunks * BK_BINS and its bin starts at r * (BK_BINS + 1).
+  uint32_t n;            // elements in a row
   uint32_t n_split;      // splitters in use
   uint32_t oversample;   // samples per bin (BK_OVERSAMPLE at most)
   uint32_t tile, tiles_per_chunk, n_chunks, chunks_per_slab, n_slabs;
@@ -72,6 +76,40 @@ struct BucketParams {
   // NULL: the path runs unconditionally.
   uint32_t* flags;
   int attempt;           // 0: not an attempt; 1: only with few distinct sample keys; 2: always
+};
+
+// The kernels' view of one row: every pointer of the parameters moved to that row (the
+// parameters themselves stay untouched in the kernel's argument segment).
+template <typename KeyT, typename PayT>
+struct BucketRow {
+  const KeyT* keys_in;
+  const int64_t* pay_in;
+  KeyT* keys_out;
+  int64_t* pay_out;
+  KeyT* buf_keys0;
+  KeyT* buf_keys1;
+  PayT* buf_pay0;
+  PayT* buf_pay1;
+  KeyT* splitters;
+  uint32_t* slab_tot;
+  uint32_t* chunk_hist;
+  uint32_t* bin_start;
+  __device__ __forceinline__ BucketRow(const BucketParams& p, uint32_t row)
+  {
+    const size_t e0 = (size_t)row * p.n;
+    keys_in    = static_cast<const KeyT*>(p.keys_in) + e0;
+    pay_in     = p.pay_in ? static_cast<const int64_t*>(p.pay_in) + e0 : nullptr;
+    keys_out   = p.keys_out ? static_cast<KeyT*>(p.keys_out) + e0 : nullptr;
+    pay_out    = p.pay_out ? static_cast<int64_t*>(p.pay_out) + e0 : nullptr;
+    buf_keys0  = static_cast<KeyT*>(p.buf_keys[0]) + e0;
+    buf_keys1  = static_cast<KeyT*>(p.buf_keys[1]) + e0;
+    buf_pay0   = p.buf_pay[0] ? static_cast<PayT*>(p.buf_pay[0]) + e0 : nullptr;
+    buf_pay1   = p.buf_pay[1] ? static_cast<PayT*>(p.buf_pay[1]) + e0 : nullptr;
+    splitters  = static_cast<KeyT*>(p.splitters) + (size_t)row * BK_SLOTS;
+    slab_tot   = p.slab_tot + (size_t)row * p.n_slabs * BK_BINS;
+    chunk_hist = p.chunk_hist + (size_t)row * p.n_chunks * BK_BINS;
+    bin_start  = p.bin_start + (size_t)row * (BK_BINS + 1);
+  }
 };
 
 // Rank of this lane's key among the keys with the same digit value that the wavefront has
@@ -284,12 +322,13 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
   constexpr int NT = BK_PLAN_NT, IPT = BK_PLAN_IPT;
   __shared__ BlockSortSmem<KeyT, uint32_t, false, NT, IPT> sm;
   const int tid = threadIdx.x;
-  for (uint32_t i = tid; i < p.n_slabs * BK_BINS; i += NT) p.slab_tot[i] = 0;
+  const BucketRow<KeyT, uint32_t> r(p, blockIdx.x);  // one workgroup per row (the payload is not touched)
+  for (uint32_t i = tid; i < p.n_slabs * BK_BINS; i += NT) r.slab_tot[i] = 0;
   // sample e of S comes from its own stretch of n / S elements, at a place inside it that a hash
   // of e picks (evenly spaced places would meet periodic data at the same phase every time)
   const uint32_t S     = (p.n_split + 1) * p.oversample;  // <= NT * IPT
   const uint32_t span  = p.n / S > 0 ? p.n / S : 1;
-  const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
+  const KeyT* in       = r.keys_in;
   const BlockSortGeom g = block_sort_geom<NT>(S);
   KeyT k[IPT];
   uint32_t nopay[1];
@@ -331,7 +370,7 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
   block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
                                                    (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, sm.vary);
   // the sorted sample is still in sm.keys; splitter t = the last sample of stretch t
-  KeyT* spl = reinterpret_cast<KeyT*>(p.splitters);
+  KeyT* spl = r.splitters;
   if (p.attempt) {
     // an attempt on a long row: if the sample holds at most 255 distinct keys, those are the
     // splitters, each with a bin of equal keys behind it
@@ -382,14 +421,15 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
   __shared__ SplitterTable<KeyT> tab;
   __shared__ uint32_t hist[NW * BK_BINS];
   if (p.flags && p.flags[0] == 0) return;  // an attempt that the plan kernel called off
+  const BucketRow<KeyT, uint32_t> r(p, blockIdx.y);
   const int tid = threadIdx.x, wave = tid >> 6;
   for (int i = tid; i < NW * BK_BINS; i += NT) hist[i] = 0;
-  load_splitters<KeyT, NT>(tab, reinterpret_cast<const KeyT*>(p.splitters));
+  load_splitters<KeyT, NT>(tab, r.splitters);
   const uint32_t chunk = blockIdx.x;
   const uint64_t clen  = (uint64_t)p.tiles_per_chunk * p.tile;
   const uint64_t b0    = (uint64_t)chunk * clen;
   const uint64_t b1    = b0 + clen < p.n ? b0 + clen : p.n;
-  const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
+  const KeyT* in       = r.keys_in;
   uint32_t* my         = hist + wave * BK_BINS;
   // (rounds of U independent loads per thread; the next round is asked for before this one is
   // searched, U searches side by side)
@@ -424,8 +464,8 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
     }
   }
   __syncthreads();
-  uint32_t* out  = p.chunk_hist + (uint64_t)chunk * BK_BINS;
-  uint32_t* slab = p.slab_tot + (uint64_t)(chunk / p.chunks_per_slab) * BK_BINS;
+  uint32_t* out  = r.chunk_hist + (uint64_t)chunk * BK_BINS;
+  uint32_t* slab = r.slab_tot + (uint64_t)(chunk / p.chunks_per_slab) * BK_BINS;
   for (int b = tid; b < BK_BINS; b += NT) {
     uint32_t c = 0;
 #pragma unroll
@@ -455,10 +495,11 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
   __shared__ uint16_t sbin[TILE];
 
   if (p.flags && p.flags[0] == 0) return;  // an attempt that the plan kernel called off
+  const BucketRow<KeyT, PayT> r(p, blockIdx.y);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t wbase = (uint32_t)wave * (64 * IPT) + lane;
   const uint32_t chunk = blockIdx.x;
-  const KeyT* in       = reinterpret_cast<const KeyT*>(p.keys_in);
+  const KeyT* in       = r.keys_in;
   const uint32_t tile0 = chunk * p.tiles_per_chunk;
   const uint32_t tiles = (p.n + TILE - 1) / TILE;
   uint32_t tile_end    = tile0 + p.tiles_per_chunk;
@@ -474,12 +515,12 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     for (int i = 0; i < IPT; ++i) {
       const uint32_t e = wbase + i * 64;
       el[i]            = in[t0 + (e < valid ? e : 0u)];
-      if constexpr (PAY == PAY_I64) pv[i] = reinterpret_cast<const int64_t*>(p.pay_in)[t0 + (e < valid ? e : 0u)];
+      if constexpr (PAY == PAY_I64) pv[i] = r.pay_in[t0 + (e < valid ? e : 0u)];
       if constexpr (PAY == PAY_IDX32) pv[i] = t0 + e;
     }
   };
   if (tile0 < tile_end) load_tile(tile0);
-  load_splitters<KeyT, NT>(tab, reinterpret_cast<const KeyT*>(p.splitters));
+  load_splitters<KeyT, NT>(tab, r.splitters);
 
   // ---- where this chunk's elements of every bin start: the bins before (all chunks), the
   // same bin in the slabs before this chunk's and in the chunks before it inside its slab
@@ -488,11 +529,11 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     if (tid < BK_BINS) {
       const uint32_t slab = chunk / p.chunks_per_slab;
       for (uint32_t s = 0; s < p.n_slabs; ++s) {
-        const uint32_t v = p.slab_tot[(uint64_t)s * BK_BINS + tid];
+        const uint32_t v = r.slab_tot[(uint64_t)s * BK_BINS + tid];
         tot += v;
         if (s < slab) before += v;
       }
-      for (uint32_t c = slab * p.chunks_per_slab; c < chunk; ++c) before += p.chunk_hist[(uint64_t)c * BK_BINS + tid];
+      for (uint32_t c = slab * p.chunks_per_slab; c < chunk; ++c) before += r.chunk_hist[(uint64_t)c * BK_BINS + tid];
     }
     const uint32_t incl = wave_incl_scan_u32(tot);
     if (tid < BK_BINS && lane == 63) wave_tot[wave] = incl;
@@ -518,17 +559,17 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
       for (int w = 0; w < wave; ++w) start += wave_tot[w];
       gpos[tid] = start + before;
       if (chunk == 0) {
-        p.bin_start[tid] = start;
-        if (tid == BK_BINS - 1) p.bin_start[BK_BINS] = p.n;
+        r.bin_start[tid] = start;
+        if (tid == BK_BINS - 1) r.bin_start[BK_BINS] = p.n;
       }
     }
     __syncthreads();
   }
 
-  KeyT* kbuf       = reinterpret_cast<KeyT*>(p.buf_keys[0]);
-  PayT* pbuf       = reinterpret_cast<PayT*>(p.buf_pay[0]);
-  KeyT* kout       = reinterpret_cast<KeyT*>(p.keys_out);
-  int64_t* pout    = reinterpret_cast<int64_t*>(p.pay_out);
+  KeyT* kbuf       = r.buf_keys0;
+  PayT* pbuf       = r.buf_pay0;
+  KeyT* kout       = r.keys_out;
+  int64_t* pout    = r.pay_out;
   uint32_t* my_hist = whist + wave * BK_BINS;
 
   for (uint32_t t = tile0; t < tile_end; ++t) {
@@ -613,7 +654,8 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
 // this path although it is longer than the path is meant for.
 template <typename KeyT, int PAY, int IPT>
 __device__ __forceinline__ void bucket_sort_long(
-  const BucketParams& p, uint32_t start, uint32_t len, KeyT base, int nbits, int xform, uint32_t* whist,
+  const BucketParams& p,
+  const BucketRow<KeyT, typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type>& r, uint32_t start, uint32_t len, KeyT base, int nbits, int xform, uint32_t* whist,
   uint32_t* wave_tot, KeyT* skeys,
   typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type* spay, uint32_t* gbase /* RADIX */,
   uint32_t* tbase /* RADIX */)
@@ -627,8 +669,8 @@ __device__ __forceinline__ void bucket_sort_long(
   uint32_t* my_hist    = whist + wave * RADIX;
   const uint32_t dv    = tid & (RADIX - 1);
   const int grp        = wave / (RADIX / 64);
-  KeyT* kout           = reinterpret_cast<KeyT*>(p.keys_out);
-  int64_t* pout        = reinterpret_cast<int64_t*>(p.pay_out);
+  KeyT* kout           = r.keys_out;
+  int64_t* pout        = r.pay_out;
   const bool is_float  = xform == XF_FLOAT;
   const KeyT flip      = xform == XF_SIGNED ? (KeyT)((KeyT)1 << (sizeof(KeyT) * 8 - 1)) : (KeyT)0;
   auto key_of = [&](KeyT raw) { return (KeyT)((is_float ? float_to_key(raw) : (KeyT)(raw ^ flip)) - base); };
@@ -638,10 +680,10 @@ __device__ __forceinline__ void bucket_sort_long(
   for (int ps = 0; ps < npass; ++ps) {
     const int shift  = ps * RADIX_BITS;
     const bool last  = ps == npass - 1;
-    const KeyT* ksrc = reinterpret_cast<const KeyT*>(p.buf_keys[cur]) + start;
-    const PayT* psrc = reinterpret_cast<const PayT*>(p.buf_pay[cur]) + start;
-    KeyT* kdst       = reinterpret_cast<KeyT*>(p.buf_keys[cur ^ 1]) + start;
-    PayT* pdst       = reinterpret_cast<PayT*>(p.buf_pay[cur ^ 1]) + start;
+    const KeyT* ksrc = (cur ? r.buf_keys1 : r.buf_keys0) + start;
+    const PayT* psrc = (cur ? r.buf_pay1 : r.buf_pay0) + start;
+    KeyT* kdst       = (cur ? r.buf_keys0 : r.buf_keys1) + start;
+    PayT* pdst       = (cur ? r.buf_pay0 : r.buf_pay1) + start;
     // ---- where every digit value starts in the bin: one read of the bin counts this pass's
     // digit, every wavefront in counters of its own (atomics of several wavefronts on the same
     // few words wait for one another), eight loads per thread in flight ----
@@ -775,14 +817,15 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   __shared__ uint32_t gbase[RADIX];
   __shared__ uint32_t tbase[RADIX];
   if (p.flags && p.flags[1] == 0) return;  // an attempt that did not go through
+  const BucketRow<KeyT, PayT> r(p, blockIdx.y);
   const int tid = threadIdx.x;
   const uint32_t g     = blockIdx.x;
-  const uint32_t start = p.bin_start[2 * g], mid = p.bin_start[2 * g + 1], end = p.bin_start[2 * g + 2];
+  const uint32_t start = r.bin_start[2 * g], mid = r.bin_start[2 * g + 1], end = r.bin_start[2 * g + 2];
   const uint32_t len   = mid - start;
-  const KeyT* kbuf     = reinterpret_cast<const KeyT*>(p.buf_keys[0]);
-  const PayT* pbuf     = reinterpret_cast<const PayT*>(p.buf_pay[0]);
-  KeyT* kout           = reinterpret_cast<KeyT*>(p.keys_out);
-  int64_t* pout        = reinterpret_cast<int64_t*>(p.pay_out);
+  const KeyT* kbuf     = r.buf_keys0;
+  const PayT* pbuf     = r.buf_pay0;
+  KeyT* kout           = r.keys_out;
+  int64_t* pout        = r.pay_out;
   auto emit = [&](uint32_t dst, KeyT el, PayT pv) {
     if (kout) kout[dst] = el;
     if constexpr (PAY == PAY_IDX32) pout[dst] = (int64_t)pv + p.index_offset;
@@ -794,14 +837,14 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   if (len == 0) return;
   // the keys of the bin lie strictly between the splitters lo and hi: sorted by key - lo, which
   // is below hi - lo and so has that many bits at most
-  const KeyT* spl = reinterpret_cast<const KeyT*>(p.splitters);
+  const KeyT* spl = r.splitters;
   const KeyT lo   = g > 0 ? spl[g - 1] : (KeyT)0;
   const KeyT hi   = spl[g];
   const unsigned long long diff = (unsigned long long)(KeyT)(hi - lo);
   const int nbits = diff ? 64 - __builtin_clzll(diff) : 0;
   const int xform = p.keys_travel ? (int)XF_UNSIGNED : p.xform;
   if (len > p.cap) {
-    bucket_sort_long<KeyT, PAY, (IPT < 8 ? IPT : 8)>(p, start, len, lo, nbits > 0 ? nbits : 1, xform, sm.whist, sm.wave_tot, sm.keys,
+    bucket_sort_long<KeyT, PAY, (IPT < 8 ? IPT : 8)>(p, r, start, len, lo, nbits > 0 ? nbits : 1, xform, sm.whist, sm.wave_tot, sm.keys,
                                      sm.pay, gbase, tbase);
     return;
   }

@@ -351,6 +351,11 @@ constexpr int bucket_sort_ipt(int kb, int pay) { return kb + pay_bytes_of(pay) <
 // tiles, and tiles as large as the staging area in LDS allows (element, payload, 2 bytes for the
 // bin) beyond that.
 constexpr int kBucketScatterIptSmall = 4;
+// chunks (workgroups) of the count and scatter kernels at most: one per CU for the medium
+// rows the path is built for (2^21 int32: 75 us with 256 chunks, 78 with 512); four per CU
+// where it is tried on long rows, so that two workgroups of the count kernel are resident per
+// CU and cover each other's waits (count of 2^28 int64: 0.69 -> 0.55 ms)
+constexpr size_t kBucketMaxChunks = 256, kBucketMaxChunksLong = 1024;
 constexpr int bucket_scatter_ipt_large(int kb, int pay)
 {
   return kb + pay_bytes_of(pay) <= 4 ? 16 : (kb + pay_bytes_of(pay) <= 12 ? 8 : 4);
@@ -424,7 +429,7 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.has_indices_in    = true;
   }
 
-  if (pl.strategy == S_RADIX && pl.rows == 1 && pl.dt.bytes <= 8 && !pl.gather_values && opt.bucket_path != 0 &&
+  if (pl.strategy == S_RADIX && pl.rows <= 65535 && pl.dt.bytes <= 8 && !pl.gather_values && opt.bucket_path != 0 &&
       (opt.target_chunks == 0 || opt.bucket_path > 0)) {  // (a chunk count is a request to the radix path)
     // One row of up to about a million elements: four launches in all instead of two per digit.
     // The bins average a quarter of what the bin sort holds in registers (sample splitters:
@@ -434,8 +439,16 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     // (up to 256 bins of half of what the registers hold on average: with 16 samples per bin a
     // bin twice the average is a one-in-a-thousand event, and such a bin is still sorted, by
     // the slower loop through global memory)
-    const size_t max_len = opt.bucket_path > 0 ? (size_t)0xFFFFFFFFu / 2 : 128 * cap;
-    if (pl.row_len <= max_len && cap >= 64) {
+    // (Several rows side by side while all of them together stay within that length: the bin
+    // sort is built for latency, one workgroup of 1024 threads per CU and bin, and beyond about
+    // one round of bins over the CUs the radix passes move more keys per second.)
+    // (4-byte keys with positions: level with the radix passes at 2^21 elements, behind them
+    // beyond, so the path ends at three quarters of that)
+    const size_t max_len = opt.bucket_path > 0 ? (size_t)0xFFFFFFFFu / 2
+                           : (pl.dt.bytes <= 4 && pl.pay != PAY_NONE ? 96 : 128) * cap;
+    // (several rows of 4-byte keys with positions: level with the radix passes at 2^20 in all)
+    const size_t max_vol = pl.rows == 1 ? max_len : pl.dt.bytes <= 4 && pl.pay != PAY_NONE ? max_len / 2 : max_len;
+    if (pl.row_len <= max_len && pl.volume <= max_vol && cap >= 64) {
       size_t bins = opt.bucket_bins ? opt.bucket_bins : (pl.row_len + 1023) / 1024;
       if (bins < 2) bins = 2;
       if (bins > 256) bins = 256;
@@ -455,23 +468,23 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
   };
 
   // chunks of the count and scatter kernels of the four-launch path, and its tables
-  auto bucket_tables = [&] {
+  auto bucket_tables = [&](size_t max_chunks) {
     pl.bk_tile            = BK_NT * (pl.row_len <= ((size_t)1 << 21) ? kBucketScatterIptSmall
                                                                        : bucket_scatter_ipt_large(pl.dt.bytes, pl.pay));
     const size_t tiles    = (pl.row_len + pl.bk_tile - 1) / pl.bk_tile;
-    const size_t want     = tiles < 256 ? tiles : 256;
+    const size_t want     = tiles < max_chunks ? tiles : max_chunks;
     pl.bk_tiles_per_chunk = (uint32_t)((tiles + want - 1) / want);
     pl.bk_chunks          = (uint32_t)((tiles + pl.bk_tiles_per_chunk - 1) / pl.bk_tiles_per_chunk);
     pl.bk_slabs           = (uint32_t)((pl.bk_chunks + kChunksPerSlab - 1) / kChunksPerSlab);
-    pl.off_bk_splitters   = take(BK_SLOTS * 8);
-    pl.off_bk_slab_tot    = take((size_t)pl.bk_slabs * BK_BINS * sizeof(uint32_t));
-    pl.off_bk_chunk_hist  = take((size_t)pl.bk_chunks * BK_BINS * sizeof(uint32_t));
-    pl.off_bk_bin_start   = take((BK_BINS + 1) * sizeof(uint32_t));
+    pl.off_bk_splitters   = take(pl.rows * BK_SLOTS * 8);
+    pl.off_bk_slab_tot    = take(pl.rows * pl.bk_slabs * BK_BINS * sizeof(uint32_t));
+    pl.off_bk_chunk_hist  = take(pl.rows * pl.bk_chunks * BK_BINS * sizeof(uint32_t));
+    pl.off_bk_bin_start   = take(pl.rows * (BK_BINS + 1) * sizeof(uint32_t));
     pl.off_bk_flags       = take(2 * sizeof(uint32_t));
   };
 
   if (pl.strategy == S_BUCKET) {
-    bucket_tables();
+    bucket_tables(kBucketMaxChunks);
     for (int b = 0; b < 2; ++b) pl.off_keys[b] = take(pl.volume * pl.dt.bytes);
     if (pl.pay != PAY_NONE)
       for (int b = 0; b < 2; ++b) pl.off_pay[b] = take(pl.volume * (pl.pay == PAY_IDX32 ? 4 : 8));
@@ -568,7 +581,7 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
       pl.low_card = opt.low_cardinality == 2 ? 2 : 1;
       pl.bk_split = BK_SLOTS - 1;
       pl.bk_cap   = (uint32_t)(BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay));
-      bucket_tables();
+      bucket_tables(kBucketMaxChunksLong);
     }
   } else if (pl.strategy == S_COUNT16) {
     // one histogram workgroup per CU and half of the key range, a few rounds of them
@@ -944,23 +957,25 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int 
   p.direct_equal    = (a.values_out == nullptr || a.values_out != a.values_in) &&
                       (a.indices_out == nullptr || a.indices_out != a.indices_in);
   constexpr int IPT = bucket_sort_ipt(sizeof(KeyT), PAY);
+  const unsigned rows = (unsigned)pl.rows;
   L.run(K_BUCKET_PLAN, [&] {
-    hipLaunchKernelGGL((bucket_plan_kernel<KeyT>), dim3(1), dim3(BK_PLAN_NT), 0, L.stream, p);
+    hipLaunchKernelGGL((bucket_plan_kernel<KeyT>), dim3(rows), dim3(BK_PLAN_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_COUNT, [&] {
-    hipLaunchKernelGGL((bucket_count_kernel<KeyT>), dim3(pl.bk_chunks), dim3(BK_COUNT_NT), 0, L.stream, p);
+    hipLaunchKernelGGL((bucket_count_kernel<KeyT>), dim3(pl.bk_chunks, rows), dim3(BK_COUNT_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_SCATTER, [&] {
     constexpr int LARGE = bucket_scatter_ipt_large(sizeof(KeyT), PAY);
     if (pl.bk_tile == (uint32_t)BK_NT * kBucketScatterIptSmall)
-      hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, kBucketScatterIptSmall>), dim3(pl.bk_chunks),
+      hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, kBucketScatterIptSmall>), dim3(pl.bk_chunks, rows),
                          dim3(BK_NT), 0, L.stream, p);
     else
-      hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, LARGE>), dim3(pl.bk_chunks), dim3(BK_NT), 0, L.stream, p);
+      hipLaunchKernelGGL((bucket_scatter_kernel<KeyT, PAY, LARGE>), dim3(pl.bk_chunks, rows), dim3(BK_NT), 0,
+                         L.stream, p);
   });
   L.run(K_BUCKET_SORT, [&] {
-    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(attempt ? BK_SLOTS : pl.bk_split + 1), dim3(BK_NT),
-                       0, L.stream, p);
+    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(attempt ? BK_SLOTS : pl.bk_split + 1, rows),
+                       dim3(BK_NT), 0, L.stream, p);
   });
 }
 

@@ -134,13 +134,17 @@ def _select_rows(a: ndarray, k: int, want_next: bool):
     return [o.to_torch().reshape(shape) for o in outs]
 
 
-def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool):
+def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool, exact_bits: bool = False):
     """``a`` has the reduction axis last: the samples at the sorted positions ``wanted`` of
     every row, as tensors of the row shape, and (or None) which rows hold a NaN.  A few
     positions on long rows are found by selection, one call per position or adjacent pair: two
     reads of the rows each instead of a sort (which moves them once or twice per key byte), and
     the rows' largest element, which comes with it, tells the NaNs.  Anything else sorts the
-    rows."""
+    rows.  The selection hands floating-point samples back as their keys keep them (a zero as
+    +0): ``exact_bits`` (the methods that return a sample itself) keeps floating-point rows on
+    the sort, so that the sample carries the bit pattern the sorted row has at that position
+    whatever the row length.  ``overwrite_input`` permits the sort to run in place; the
+    selection leaves the input as it is, which the permission covers."""
     from .module import sort
 
     n = a.shape[-1]
@@ -153,7 +157,7 @@ def _order_statistics(a: ndarray, wanted: Sequence[int], overwrite_input: bool):
             pairs.append((k, False))
     # a selection costs about two reads of the rows, a sort two (one read, one write) per key byte
     if (0 < len(pairs) <= a.dtype.itemsize // 2 + 1 and n >= (1 << 16) and a.dtype.itemsize >= 4 and
-            a.dtype.kind in "fiu" and a.size):
+            a.dtype.kind in "fiu" and a.size and not (exact_bits and a.dtype.kind == "f")):
         out: dict[int, torch.Tensor] = {}
         top = None
         for k, with_next in pairs:
@@ -236,7 +240,7 @@ def quantile(a: Any, q: Any, axis: Union[None, int, Iterable[int]] = None, out: 
     # ---- the samples around every quantile ---------------------------------------------
     places = [_position(method, float(qv), n) for qv in q_arr.reshape(-1)]
     wanted = [p[0] for p in places] + [p[1] for p in places]
-    stats, has_nan = _order_statistics(rows, wanted, overwrite_input)
+    stats, has_nan = _order_statistics(rows, wanted, overwrite_input, exact_bits=method in _SAMPLE_METHODS)
     to_dtype = a.dtype if method in _SAMPLE_METHODS else np.dtype(np.float64)
     tdt = _torch_dtype(to_dtype)
     results = []

@@ -78,6 +78,43 @@ def test_payload_in_place_offset_and_values(abi, dtype):
         assert np.array_equal(idx, pay[ref]) and bits_equal(vals, a[ref])
 
 
+@pytest.mark.parametrize("dtype", SERVED, ids=lambda d: np.dtype(d).name)
+def test_several_rows_side_by_side(abi, dtype):
+    """Rows too long for the row kernels whose total stays within the path's length: every row
+    gets its own splitters, counts and bins (second launch dimension).  Rows that differ in
+    kind (random, constant, few values, sorted), row starts that are not multiples of a line,
+    a caller's payload, in place, an index offset."""
+    rng = np.random.default_rng(77)
+    for rows, row_len in ((3, 20001), (7, 40003), (2, 300001), (30, 17001)):
+        a = random_array(dtype, rows * row_len, rng).reshape(rows, row_len)
+        a[0] = a[0, 0]
+        if rows > 2:
+            a[1] = a[1, rng.integers(0, 5, row_len)]
+            a[2] = np.sort(a[2], kind="stable")
+        plan = abi.describe_plan(dtype, a.size, row_len, True)
+        print(f"bucket rows dtype={np.dtype(dtype).name} rows={rows} row_len={row_len} plan={plan}", flush=True)
+        assert "strategy=bucket" in plan, plan
+        perm = np.argsort(a, axis=1, kind="stable")
+        got = abi.local_sort(a, row_len, argsort=True).reshape(rows, row_len)
+        assert np.array_equal(got, perm)
+        vals = abi.local_sort(a, row_len, argsort=False).reshape(rows, row_len)
+        assert bits_equal(vals, np.take_along_axis(a, perm, axis=1))
+        assert bits_equal(abi.local_sort(a, row_len, argsort=False, inplace=True).reshape(rows, row_len),
+                          np.take_along_axis(a, perm, axis=1))
+        assert np.array_equal(abi.local_sort(a, row_len, argsort=True, index_offset=7).reshape(rows, row_len), perm + 7)
+        pay = rng.integers(-2**62, 2**62, a.size, dtype=np.int64)
+        want = np.take_along_axis(pay.reshape(rows, row_len), perm, axis=1)
+        for inplace in (False, True):
+            got = abi.local_sort(a, row_len, argsort=True, indices_in=pay, inplace=inplace).reshape(rows, row_len)
+            assert np.array_equal(got, want)
+        assert np.array_equal(abi.local_sort(a, row_len, argsort=True), oracle.local_sort(a.reshape(-1), row_len, True))
+
+
+def test_rows_beyond_the_paths_total_take_the_radix_passes(abi):
+    assert "strategy=radix" in abi.describe_plan(np.int32, 64 << 20, 1 << 20, True)
+    assert "strategy=bucket" in abi.describe_plan(np.int32, 2 << 20, 1 << 20, False)
+
+
 def adversarial(kind, n, rng):
     if kind == "sorted":
         return np.sort(rng.integers(-2**31, 2**31, n, dtype=np.int64)).astype(np.int32)
