@@ -40,7 +40,7 @@ static constexpr int kMaxDevices = 64;
 // misort_init): ballots if the environment says MISORT_RANK_BALLOT=1 (read once), ballots on
 // anything that is not gfx950, and otherwise a short probe on a stream of its own (three
 // launches of lds_lane_order_probe_kernel, 25 million lane operations with 256, 4 and 1
-// distinct words per wavefront, about 0.1 ms) that compares the returning add with the ballot
+// distinct words per wavefront, about 0.35 ms) that compares the returning add with the ballot
 // match lane by lane: adds only if not one lane disagrees.  The verdict is kept per GPU.
 enum RankMode : int { RANK_UNTESTED = 0, RANK_ADD = 1, RANK_BALLOT = 2 };
 static std::atomic<int> g_rank_mode[kMaxDevices];

@@ -308,7 +308,7 @@ int misort_init(void);
  * LDS add per key, 2 = wave ballots, 0 = not decided yet (no sort has run here and
  * misort_init was not called).  The adds are stable only where the LDS serves the lanes of
  * one instruction that hit the same word in ascending lane order; the library uses them only
- * on gfx950 and only after a probe of 25 million lane operations on that GPU (about 0.1 ms,
+ * on gfx950 and only after a probe of 25 million lane operations on that GPU (about 0.35 ms,
  * on a stream of its own, once per GPU and process) has found every lane in order, and
  * MISORT_RANK_BALLOT=1 in the environment rules them out.  No counterpart in the reference.
  */
