@@ -848,23 +848,36 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
                                      sm.pay, gbase, tbase);
     return;
   }
+  // The bin in registers, in the instantiation for exactly its number of rows per wavefront:
+  // the slots of a wider one would stay live through the passes, and at 16 slots of 8 bytes
+  // that costs registers the passes need (144 bytes per lane in scratch memory).
   const BlockSortGeom geo = block_sort_geom<NT>(len);
-  KeyT el[IPT];
-  PayT pv[HAS_PAY ? IPT : 1];
+  auto in_registers = [&](auto rows_tag) {
+    constexpr int RR = decltype(rows_tag)::value;
+    KeyT el[RR];
+    PayT pv[HAS_PAY ? RR : 1];
 #pragma unroll
-  for (int i = 0; i < IPT; ++i) {
-    const uint32_t e = geo.wbase + i * 64;
-    if ((uint32_t)i < geo.R && e < len) {
-      el[i] = kbuf[start + e];
-      if constexpr (HAS_PAY) pv[i] = pbuf[start + e];
+    for (int i = 0; i < RR; ++i) {
+      const uint32_t e = geo.wbase + i * 64;
+      if (e < len) {
+        el[i] = kbuf[start + e];
+        if constexpr (HAS_PAY) pv[i] = pbuf[start + e];
+      }
     }
-  }
-  block_radix_sort<KeyT, PayT, HAS_PAY, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, el, pv, len, lo, nbits,
-                                                 xform, p.rank_by_add);
+    block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, RR, RR>(sm.whist, sm.wave_tot, sm.keys, sm.pay, el, pv, len, lo,
+                                                           nbits, xform, p.rank_by_add, ~0ull);
 #pragma unroll
-  for (int i = 0; i < IPT; ++i) {
-    const uint32_t e = geo.wbase + i * 64;
-    if ((uint32_t)i < geo.R && e < len) emit(start + e, el[i], HAS_PAY ? pv[HAS_PAY ? i : 0] : PayT{});
+    for (int i = 0; i < RR; ++i) {
+      const uint32_t e = geo.wbase + i * 64;
+      if (e < len) emit(start + e, el[i], HAS_PAY ? pv[HAS_PAY ? i : 0] : PayT{});
+    }
+  };
+  if (geo.R == 1) in_registers(std::integral_constant<int, 1>{});
+  else if (geo.R == 2) in_registers(std::integral_constant<int, 2>{});
+  else if (geo.R == 4) in_registers(std::integral_constant<int, 4>{});
+  else if constexpr (IPT >= 8) {
+    if (geo.R == 8) in_registers(std::integral_constant<int, 8>{});
+    else if constexpr (IPT >= 16) in_registers(std::integral_constant<int, 16>{});
   }
 }
 

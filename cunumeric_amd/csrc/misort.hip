@@ -142,6 +142,8 @@ struct PlanOptions {
   int low_cardinality = -1;             // long rows try the four-launch path first: < 0: rows of 2^27 elements
                                         // and more, where the sample holds few distinct keys; 0: never;
                                         // 1: the same for every length; 2: with any sample
+  int counting_sort = -1;               // one row of 2-byte values: < 0: counted from the built-in length on;
+                                        // 0: never; > 0: whenever the row is too long for the row kernels
 };
 
 static int fail(int code, const std::string& msg)
@@ -369,8 +371,12 @@ static constexpr size_t kTargetChunks  = 512;
 static constexpr size_t kChunksPerSlab = 16;
 static constexpr int kUpsweepThreads   = 256;
 static constexpr int kUpsweepDigitThreads = 256;  // upsweep over the digit side-band
-// values-only sorts of 2-byte elements: counted instead of radix-sorted from this length on
-static constexpr size_t kCount16MinLen = (size_t)1 << 20;
+// values-only sorts of one row of 2-byte elements: counted instead of radix-sorted from this
+// length on (two radix passes are ahead below: uniform int16 at 2^24 120 us against 195, level
+// near 2^25.5; float16, whose radix sort also restores -0 and NaN payloads, 148 against 111 at
+// 2^24, level near 2^23.5)
+static constexpr size_t kCount16MinLenInt   = (size_t)1 << 26;
+static constexpr size_t kCount16MinLenFloat = (size_t)1 << 24;
 static constexpr size_t kCount16Chunks = 512;
 
 // target_chunks: chunks (workgroups) a radix pass over the whole array is cut into; 0 = the
@@ -414,7 +420,9 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
   } else if (rowsort_supported(pl.dt.bytes, pl.row_len, pl.pay, pl.gather_values) &&
              pl.row_len <= rowsort_block_max(pl.dt.bytes, pl.pay)) {
     pl.strategy = S_ROW_BLOCK;
-  } else if (pl.dt.bytes == 2 && pl.pay == PAY_NONE && pl.rows == 1 && pl.row_len >= kCount16MinLen) {
+  } else if (pl.dt.bytes == 2 && pl.pay == PAY_NONE && pl.rows == 1 && opt.counting_sort != 0 &&
+             (opt.counting_sort > 0 ||
+              pl.row_len >= (pl.dt.xform == XF_FLOAT ? kCount16MinLenFloat : kCount16MinLenInt))) {
     pl.strategy = S_COUNT16;
   } else if (pl.dt.bytes == 1 && pl.pay == PAY_NONE && pl.rows == 1) {
     pl.strategy = S_COUNT8;  // any single row too long for the row kernels
@@ -431,23 +439,31 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
 
   if (pl.strategy == S_RADIX && pl.rows <= 65535 && pl.dt.bytes <= 8 && !pl.gather_values && opt.bucket_path != 0 &&
       (opt.target_chunks == 0 || opt.bucket_path > 0)) {  // (a chunk count is a request to the radix path)
-    // One row of up to about a million elements: four launches in all instead of two per digit.
-    // The bins average a quarter of what the bin sort holds in registers (sample splitters:
-    // a bin four times the average does not happen), and there are at most 256 of them.
-    const size_t cap = opt.bucket_cap ? std::min<size_t>(opt.bucket_cap, (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay))
-                                      : (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay);
-    // (up to 256 bins of half of what the registers hold on average: with 16 samples per bin a
-    // bin twice the average is a one-in-a-thousand event, and such a bin is still sorted, by
-    // the slower loop through global memory)
-    // (Several rows side by side while all of them together stay within that length: the bin
-    // sort is built for latency, one workgroup of 1024 threads per CU and bin, and beyond about
-    // one round of bins over the CUs the radix passes move more keys per second.)
-    // (4-byte keys with positions: level with the radix passes at 2^21 elements, behind them
-    // beyond, so the path ends at three quarters of that)
-    const size_t max_len = opt.bucket_path > 0 ? (size_t)0xFFFFFFFFu / 2
-                           : (pl.dt.bytes <= 4 && pl.pay != PAY_NONE ? 96 : 128) * cap;
-    // (several rows of 4-byte keys with positions: level with the radix passes at 2^20 in all)
-    const size_t max_vol = pl.rows == 1 ? max_len : pl.dt.bytes <= 4 && pl.pay != PAY_NONE ? max_len / 2 : max_len;
+    // Rows of up to about two million elements: four launches in all instead of two per digit.
+    const size_t cap_full = (size_t)BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay);
+    const size_t cap      = opt.bucket_cap ? std::min<size_t>(opt.bucket_cap, cap_full) : cap_full;
+    // Up to 256 bins of half of what the registers hold on average: with 16 samples per bin a
+    // bin twice the average is a one-in-a-thousand event, and such a bin is still sorted, by the
+    // slower loop through global memory.  Where the path ends is measured against the radix
+    // passes (random keys, back to back): 4-byte keys are ahead up to 2^21 elements in one row
+    // (72 us against 92; 131 against 99 at 3 x 2^20), 8-byte keys as far as the bins fit (108
+    // against 202 at 2^21), 2-byte keys, which take two radix passes only, up to 2^19 alone
+    // (37 against 40; float16, whose radix sort patches zeros and NaNs afterwards, 2^20) and 2^18
+    // with positions, 1-byte keys nowhere (one radix pass: 17-20 us against 21-41).  Several rows
+    // side by side while all of them together stay within a length of the same kind: the bin
+    // sort is built for latency, one workgroup of 1024 threads per CU and bin, and beyond one or
+    // two rounds of bins over the CUs the radix passes move more keys per second (8 rows of
+    // int32 at 2^21 in all: 98 against 93; 8-byte keys ahead up to 2^22: 211 against 264 alone,
+    // 224 against 329 with positions).
+    const bool forced = opt.bucket_path > 0;
+    size_t max_len = 128 * cap_full, max_vol = 128 * cap_full;
+    if (pl.dt.bytes == 8) max_vol = (size_t)1 << 22;
+    if (pl.dt.bytes == 4) max_vol = 96 * cap_full;
+    if (pl.dt.bytes == 2)
+      max_len = max_vol = (pl.pay != PAY_NONE ? 16 : pl.dt.xform == XF_FLOAT ? 64 : 32) * cap_full;
+    if (pl.dt.bytes == 1) max_len = max_vol = 0;
+    if (pl.rows == 1) max_vol = max_len;
+    if (forced) max_len = max_vol = (size_t)0xFFFFFFFFu / 2;
     if (pl.row_len <= max_len && pl.volume <= max_vol && cap >= 64) {
       size_t bins = opt.bucket_bins ? opt.bucket_bins : (pl.row_len + 1023) / 1024;
       if (bins < 2) bins = 2;
@@ -974,8 +990,8 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int 
                          L.stream, p);
   });
   L.run(K_BUCKET_SORT, [&] {
-    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), dim3(attempt ? BK_SLOTS : pl.bk_split + 1, rows),
-                       dim3(BK_NT), 0, L.stream, p);
+    const dim3 grid(attempt ? BK_SLOTS : pl.bk_split + 1, rows);
+    hipLaunchKernelGGL((bucket_sort_kernel<KeyT, PAY, IPT>), grid, dim3(BK_NT), 0, L.stream, p);
   });
 }
 
@@ -1483,6 +1499,7 @@ static PlanOptions plan_options(const misort_options* o)
     opt.bucket_cap           = o->bucket_cap;
     opt.low_cardinality      = o->low_cardinality;
     opt.bucket_oversample    = o->bucket_oversample;
+    opt.counting_sort        = o->counting_sort;
   }
   return opt;
 }

@@ -254,11 +254,13 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *   target_chunks         as misort_local_chunked (0: built in)
  *   early_last_min_bytes  from how many bytes of keys on the passes over constant most
  *                         significant digits are left out as well (< 0: built in, 256 MB)
- *   bucket_path           single rows of up to about a million elements are sorted in four
- *                         launches (splitters from a sorted sample, count, scatter into at most
- *                         256 bins, radix sort of every bin inside one workgroup) instead of two
- *                         launches per digit.  < 0: built in; 0: never; > 0: for every single
- *                         row of 1- to 8-byte elements, whatever its length
+ *   bucket_path           rows of up to about two million elements (all rows of the call
+ *                         together) are sorted in four launches (splitters from a sorted sample,
+ *                         count, scatter into at most 256 bins, radix sort of every bin inside
+ *                         one workgroup) instead of two launches per digit.  < 0: built in (2-
+ *                         to 8-byte elements, up to the lengths where the radix passes catch
+ *                         up); 0: never; > 0: for all rows of 1- to 8-byte elements, whatever
+ *                         their length
  *   bucket_bins           number of bins, 2 .. 256 (0: built in, one per 1024 elements)
  *   bucket_cap            longest bin that is sorted in registers; longer ones take the
  *                         workgroup's loop through global memory (0: built in, 8192 or 16384)
@@ -272,6 +274,10 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *                         < 0: built in (rows of 2^27 elements and more: the attempt costs
  *                         35-50 us where it is called off); 0: never; 1: rows of any length;
  *                         2: tried with any sample (tests of the way back to the radix path)
+ *   counting_sort         values-only sorts of one row of 2-byte elements are counted (65536
+ *                         counters) instead of radix-sorted.  < 0: built in (from 2^24 float16
+ *                         and 2^26 integer elements on, where counting is ahead); 0: never;
+ *                         > 0: every such row that is too long for the row kernels
  */
 typedef struct misort_options {
   size_t target_chunks;
@@ -281,6 +287,7 @@ typedef struct misort_options {
   unsigned bucket_cap;
   int low_cardinality;
   unsigned bucket_oversample;
+  int counting_sort;
 } misort_options;
 size_t misort_scratch_bytes_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                                  int has_indices_in, const misort_options* options);

@@ -41,11 +41,14 @@ def test_every_dtype_over_the_sizes_the_path_serves(abi, dtype):
         for narrow in (False, True):
             a = random_array(dtype, n, rng, narrow=narrow)
             print(f"bucket dtype={np.dtype(dtype).name} n={n} narrow={narrow}", flush=True)
-            plan = abi.describe_plan(dtype, n, n, True)
+            # (1-byte keys never take the path by themselves, one radix pass being quicker,
+            # and 2-byte keys with positions up to 2^18 elements only: asked for here)
+            kw = dict(options=Options(bucket_path=1)) if np.dtype(dtype).itemsize <= 2 else {}
+            plan = abi.describe_plan(dtype, n, n, True, **kw)
             if np.dtype(dtype) != np.complex128:
                 assert "strategy=bucket" in plan, plan
-            check(abi, a)
-            assert np.array_equal(abi.local_sort(a, n, argsort=True), oracle.local_sort(a, n, True))
+            check(abi, a, **kw)
+            assert np.array_equal(abi.local_sort(a, n, argsort=True, **kw), oracle.local_sort(a, n, True))
 
 
 @pytest.mark.parametrize("dtype", [np.int32, np.float32, np.uint64, np.float64, np.complex64],
@@ -63,18 +66,19 @@ def test_a_million_elements(abi, dtype):
 def test_payload_in_place_offset_and_values(abi, dtype):
     rng = np.random.default_rng(73)
     n = 70001
+    kw = dict(options=Options(bucket_path=1)) if np.dtype(dtype).itemsize == 1 else {}
     a = random_array(dtype, n, rng)
     ref = np.argsort(a, kind="stable")
     pay = rng.integers(-2**62, 2**62, n, dtype=np.int64)
     for inplace in (False, True):
-        got = abi.local_sort(a, n, argsort=True, indices_in=pay, inplace=inplace)
+        got = abi.local_sort(a, n, argsort=True, indices_in=pay, inplace=inplace, **kw)
         assert np.array_equal(got, pay[ref])
-    assert np.array_equal(abi.local_sort(a, n, argsort=True, index_offset=12345), ref + 12345)
-    assert bits_equal(abi.local_sort(a, n, argsort=False, inplace=True), np.sort(a, kind="stable"))
-    idx, vals = abi.local_sort(a, n, argsort=True, want_values=True)
+    assert np.array_equal(abi.local_sort(a, n, argsort=True, index_offset=12345, **kw), ref + 12345)
+    assert bits_equal(abi.local_sort(a, n, argsort=False, inplace=True, **kw), np.sort(a, kind="stable"))
+    idx, vals = abi.local_sort(a, n, argsort=True, want_values=True, **kw)
     assert np.array_equal(idx, ref) and bits_equal(vals, a[ref])
     if np.dtype(dtype).kind != "c":
-        idx, vals = abi.local_sort(a, n, argsort=True, indices_in=pay, want_values=True)
+        idx, vals = abi.local_sort(a, n, argsort=True, indices_in=pay, want_values=True, **kw)
         assert np.array_equal(idx, pay[ref]) and bits_equal(vals, a[ref])
 
 
@@ -91,28 +95,42 @@ def test_several_rows_side_by_side(abi, dtype):
         if rows > 2:
             a[1] = a[1, rng.integers(0, 5, row_len)]
             a[2] = np.sort(a[2], kind="stable")
-        plan = abi.describe_plan(dtype, a.size, row_len, True)
+        kw = dict(options=Options(bucket_path=1))   # (where the path ends by itself depends on the type)
+        plan = abi.describe_plan(dtype, a.size, row_len, True, **kw)
         print(f"bucket rows dtype={np.dtype(dtype).name} rows={rows} row_len={row_len} plan={plan}", flush=True)
         assert "strategy=bucket" in plan, plan
         perm = np.argsort(a, axis=1, kind="stable")
-        got = abi.local_sort(a, row_len, argsort=True).reshape(rows, row_len)
+        got = abi.local_sort(a, row_len, argsort=True, **kw).reshape(rows, row_len)
         assert np.array_equal(got, perm)
-        vals = abi.local_sort(a, row_len, argsort=False).reshape(rows, row_len)
+        vals = abi.local_sort(a, row_len, argsort=False, **kw).reshape(rows, row_len)
         assert bits_equal(vals, np.take_along_axis(a, perm, axis=1))
-        assert bits_equal(abi.local_sort(a, row_len, argsort=False, inplace=True).reshape(rows, row_len),
+        assert bits_equal(abi.local_sort(a, row_len, argsort=False, inplace=True, **kw).reshape(rows, row_len),
                           np.take_along_axis(a, perm, axis=1))
-        assert np.array_equal(abi.local_sort(a, row_len, argsort=True, index_offset=7).reshape(rows, row_len), perm + 7)
+        assert np.array_equal(abi.local_sort(a, row_len, argsort=True, index_offset=7, **kw).reshape(rows, row_len),
+                              perm + 7)
         pay = rng.integers(-2**62, 2**62, a.size, dtype=np.int64)
         want = np.take_along_axis(pay.reshape(rows, row_len), perm, axis=1)
         for inplace in (False, True):
-            got = abi.local_sort(a, row_len, argsort=True, indices_in=pay, inplace=inplace).reshape(rows, row_len)
+            got = abi.local_sort(a, row_len, argsort=True, indices_in=pay, inplace=inplace, **kw).reshape(rows, row_len)
             assert np.array_equal(got, want)
-        assert np.array_equal(abi.local_sort(a, row_len, argsort=True), oracle.local_sort(a.reshape(-1), row_len, True))
+        assert np.array_equal(abi.local_sort(a, row_len, argsort=True, **kw),
+                              oracle.local_sort(a.reshape(-1), row_len, True))
 
 
-def test_rows_beyond_the_paths_total_take_the_radix_passes(abi):
+def test_where_the_path_ends_by_itself(abi):
+    """The built-in limits: measured against the radix passes per element size."""
+    bucket = lambda dtype, vol, row, arg: "strategy=bucket" in abi.describe_plan(dtype, vol, row, arg)
+    assert bucket(np.int32, 1 << 21, 1 << 21, False) and bucket(np.int32, 1 << 21, 1 << 21, True)
+    assert not bucket(np.int32, (1 << 21) + 1, (1 << 21) + 1, False)
+    assert bucket(np.int32, 3 << 19, 3 << 16, False) and not bucket(np.int32, 1 << 21, 1 << 18, False)
+    assert bucket(np.float64, 1 << 21, 1 << 21, False) and not bucket(np.float64, 1 << 21, 1 << 21, True)
+    assert bucket(np.int64, 1 << 22, 1 << 19, True) and not bucket(np.int64, 1 << 23, 1 << 19, True)
+    assert bucket(np.int16, 1 << 19, 1 << 19, False) and not bucket(np.int16, 1 << 20, 1 << 20, False)
+    assert bucket(np.float16, 1 << 20, 1 << 20, False)
+    assert bucket(np.int16, 1 << 18, 1 << 18, True) and not bucket(np.int16, 1 << 19, 1 << 19, True)
+    assert not bucket(np.int8, 1 << 16, 1 << 16, True) and not bucket(np.uint8, 1 << 17, 1 << 15, False)
+    assert not bucket(np.complex128, 1 << 16, 1 << 16, True)
     assert "strategy=radix" in abi.describe_plan(np.int32, 64 << 20, 1 << 20, True)
-    assert "strategy=bucket" in abi.describe_plan(np.int32, 2 << 20, 1 << 20, False)
 
 
 def adversarial(kind, n, rng):

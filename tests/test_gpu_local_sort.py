@@ -4,6 +4,7 @@ Bit-exact: sorted values byte for byte, stable-argsort indices exactly."""
 import numpy as np
 import pytest
 
+from cunumeric_amd._lib import Options
 from oracle import misort_oracle as oracle
 from tests.util import ALL_DTYPES, Abi, bits_equal, random_array
 
@@ -145,7 +146,8 @@ def test_default_plan_multi_tile_chunks(abi, dtype):
 
 @pytest.mark.parametrize("dtype", [np.int16, np.uint16, np.float16], ids=lambda d: np.dtype(d).name)
 def test_counting_sort_of_two_byte_values(abi, dtype):
-    """Long 1-D values-only sorts of 2-byte elements take the counting path."""
+    """Long 1-D values-only sorts of 2-byte elements take the counting path: by themselves
+    from 2^24 (float16) or 2^26 (integers) elements on, asked for here at a million."""
     rng = np.random.default_rng(31)
     n = (1 << 20) + 12345
     cases = {
@@ -157,10 +159,15 @@ def test_counting_sort_of_two_byte_values(abi, dtype):
     }
     for name, a in cases.items():
         print(f"count16 dtype={np.dtype(dtype).name} case={name}", flush=True)
-        assert "strategy=count16" in abi.describe_plan(a.dtype, a.size, a.size, False)
+        o = Options(counting_sort=1)
+        assert "strategy=count16" in abi.describe_plan(a.dtype, a.size, a.size, False, options=o)
         ref = np.sort(a, kind="stable")
-        assert bits_equal(abi.local_sort(a, a.size, argsort=False), ref), name
-        assert bits_equal(abi.local_sort(a, a.size, argsort=False, inplace=True), ref), name
+        assert bits_equal(abi.local_sort(a, a.size, argsort=False, options=o), ref), name
+        assert bits_equal(abi.local_sort(a, a.size, argsort=False, inplace=True, options=o), ref), name
+    assert "strategy=count16" in abi.describe_plan(np.float16, 1 << 24, 1 << 24, False)
+    assert "strategy=count16" not in abi.describe_plan(np.int16, 1 << 24, 1 << 24, False)
+    assert "strategy=count16" in abi.describe_plan(np.int16, 1 << 26, 1 << 26, False)
+    assert "strategy=count16" not in abi.describe_plan(np.int16, 1 << 26, 1 << 26, False, options=Options(counting_sort=0))
 
 
 @pytest.mark.parametrize("dtype", [np.bool_, np.int8, np.uint8], ids=lambda d: np.dtype(d).name)
