@@ -1,4 +1,4 @@
-// Sort of rows of a few ten thousand to about a million elements in four launches: sample
+// Sort of rows of a few ten thousand to about two million elements in four launches: sample
 // -> count -> scatter -> sort the bins.  It serves the sizes where the radix path's two
 // launches per digit are mostly launch and start-up time (the reference's own benchmark sorts
 // 10^6 elements, examples/sort.py:110-123; the calls replaced are the same ones,
