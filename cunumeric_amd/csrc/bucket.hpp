@@ -525,15 +525,39 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
   // ---- where this chunk's elements of every bin start: the bins before (all chunks), the
   // same bin in the slabs before this chunk's and in the chunks before it inside its slab
   {
+    // (the first half of the workgroup adds up the slabs, the second the chunks before this
+    // one in its slab, four loads in flight each: one after the other the up to 30 reads were
+    // a third of the kernel's time on short rows)
+    static_assert(NT == 2 * BK_BINS, "one thread per bin for the slabs, one for the chunks");
     uint32_t tot = 0, before = 0;
-    if (tid < BK_BINS) {
+    {
+      const uint32_t bin  = tid & (BK_BINS - 1);
       const uint32_t slab = chunk / p.chunks_per_slab;
-      for (uint32_t s = 0; s < p.n_slabs; ++s) {
-        const uint32_t v = r.slab_tot[(uint64_t)s * BK_BINS + tid];
-        tot += v;
-        if (s < slab) before += v;
+      if (tid < BK_BINS) {
+        for (uint32_t s0 = 0; s0 < p.n_slabs; s0 += 4) {
+          uint32_t v[4];
+#pragma unroll
+          for (uint32_t j = 0; j < 4; ++j)
+            v[j] = r.slab_tot[(uint64_t)(s0 + j < p.n_slabs ? s0 + j : s0) * BK_BINS + bin];
+#pragma unroll
+          for (uint32_t j = 0; j < 4; ++j)
+            if (s0 + j < p.n_slabs) {
+              tot += v[j];
+              if (s0 + j < slab) before += v[j];
+            }
+        }
+      } else {
+        uint32_t sum = 0;
+        for (uint32_t c0 = slab * p.chunks_per_slab; c0 < chunk; c0 += 4) {
+          uint32_t v[4];
+#pragma unroll
+          for (uint32_t j = 0; j < 4; ++j) v[j] = r.chunk_hist[(uint64_t)(c0 + j < chunk ? c0 + j : c0) * BK_BINS + bin];
+#pragma unroll
+          for (uint32_t j = 0; j < 4; ++j)
+            if (c0 + j < chunk) sum += v[j];
+        }
+        whist[bin] = sum;  // (whist is free until the first tile)
       }
-      for (uint32_t c = slab * p.chunks_per_slab; c < chunk; ++c) before += r.chunk_hist[(uint64_t)c * BK_BINS + tid];
     }
     const uint32_t incl = wave_incl_scan_u32(tot);
     if (tid < BK_BINS && lane == 63) wave_tot[wave] = incl;
@@ -557,7 +581,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     if (tid < BK_BINS) {
       uint32_t start = incl - tot;
       for (int w = 0; w < wave; ++w) start += wave_tot[w];
-      gpos[tid] = start + before;
+      gpos[tid] = start + before + whist[tid];
       if (chunk == 0) {
         r.bin_start[tid] = start;
         if (tid == BK_BINS - 1) r.bin_start[BK_BINS] = p.n;
@@ -575,7 +599,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
   for (uint32_t t = tile0; t < tile_end; ++t) {
     const uint32_t t0    = t * TILE;
     const uint32_t valid = p.n - t0 < (uint32_t)TILE ? p.n - t0 : (uint32_t)TILE;
-    uint32_t b[IPT], r[IPT];
+    uint32_t b[IPT], rk[IPT];
     for (int i = tid; i < NW * BK_BINS; i += NT) whist[i] = 0;
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
@@ -586,7 +610,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     lds_barrier();
     // (slots past the end of the row in the last tile hold no key)
 #pragma unroll
-    for (int i = 0; i < IPT; ++i) r[i] = wave_rank<9>(my_hist, b[i], wbase + i * 64 < valid, p.rank_by_add);
+    for (int i = 0; i < IPT; ++i) rk[i] = wave_rank<9>(my_hist, b[i], wbase + i * 64 < valid, p.rank_by_add);
     lds_barrier();
     uint32_t tot = 0;
     if (tid < BK_BINS) {
@@ -611,7 +635,7 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
 #pragma unroll
     for (int i = 0; i < IPT; ++i) {
       if (wbase + i * 64 < valid) {
-        const uint32_t q = my_hist[b[i]] + r[i];
+        const uint32_t q = my_hist[b[i]] + rk[i];
         skeys[q]         = el[i];
         if constexpr (HAS_PAY) spay[q] = pv[i];
         sbin[q] = (uint16_t)b[i];
@@ -732,12 +756,12 @@ __device__ __forceinline__ void bucket_sort_long(
     for (uint32_t t0 = 0; t0 < len; t0 += TILE) {
       const uint32_t valid = len - t0 < (uint32_t)TILE ? len - t0 : (uint32_t)TILE;
       for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;
-      uint32_t d[IPT], r[IPT];
+      uint32_t d[IPT], rk[IPT];
 #pragma unroll
       for (int i = 0; i < IPT; ++i) d[i] = KeyOps<KeyT>::digit(key_of(el[i]), shift);
       lds_barrier();
 #pragma unroll
-      for (int i = 0; i < IPT; ++i) r[i] = wave_rank<RADIX_BITS>(my_hist, d[i], wbase + i * 64 < valid, p.rank_by_add);
+      for (int i = 0; i < IPT; ++i) rk[i] = wave_rank<RADIX_BITS>(my_hist, d[i], wbase + i * 64 < valid, p.rank_by_add);
       lds_barrier();
       uint32_t count = 0, before = 0;
 #pragma unroll
@@ -765,7 +789,7 @@ __device__ __forceinline__ void bucket_sort_long(
 #pragma unroll
       for (int i = 0; i < IPT; ++i) {
         if (wbase + i * 64 < valid) {
-          const uint32_t q = my_hist[d[i]] + r[i];
+          const uint32_t q = my_hist[d[i]] + rk[i];
           skeys[q]         = el[i];
           if constexpr (HAS_PAY) spay[q] = pv[i];
         }
