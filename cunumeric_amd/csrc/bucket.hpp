@@ -211,7 +211,9 @@ __device__ __forceinline__ BlockSortGeom block_sort_geom(uint32_t len)
 
 // the passes for R = RR rows per wavefront: straight-line code over the RR slots (rows that
 // lie beyond the elements have no valid lane and do nothing)
-template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT, int RR>
+// SHARED_LDS: skeys and spay are the same memory (16384 elements of 12 or 16 bytes do not fit
+// the LDS side by side); the payload then follows the keys through it in a second step.
+template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT, int RR, bool SHARED_LDS = false>
 __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t* wave_tot, KeyT* skeys,
                                                       PayT* spay, KeyT (&el)[IPT],
                                                       PayT (&pay)[HAS_PAY ? IPT : 1], uint32_t len, KeyT base,
@@ -275,7 +277,7 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
     for (int i = 0; i < RR; ++i) {
       if (wbase + i * 64 < len) {
         skeys[q[i]] = el[i];
-        if constexpr (HAS_PAY) spay[q[i]] = pay[i];
+        if constexpr (HAS_PAY && !SHARED_LDS) spay[q[i]] = pay[i];
       }
     }
     __syncthreads();
@@ -284,8 +286,19 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
     for (int i = 0; i < RR; ++i) {
       if (wbase + i * 64 < len) {
         el[i] = skeys[wbase + i * 64];
-        if constexpr (HAS_PAY) pay[i] = spay[wbase + i * 64];
+        if constexpr (HAS_PAY && !SHARED_LDS) pay[i] = spay[wbase + i * 64];
       }
+    }
+    if constexpr (HAS_PAY && SHARED_LDS) {
+      __syncthreads();  // (every key has been read back)
+#pragma unroll
+      for (int i = 0; i < RR; ++i)
+        if (wbase + i * 64 < len) spay[q[i]] = pay[i];
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < RR; ++i)
+        if (wbase + i * 64 < len) pay[i] = spay[wbase + i * 64];
+      // (the next pass writes keys only after two more barriers)
     }
   }
 }
@@ -367,8 +380,36 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
     if ((tid & 63) == 0 && vv) atomicOr(&sm.vary, vv);
     __syncthreads();
   }
+  // 8-byte keys that vary in more than 40 bits: the passes over the 40 most significant of
+  // those bits put the sample in order unless two sample keys agree in all of them and differ
+  // below (for 4096 keys drawn from doubles or 64-bit integers a rare event: about one sample
+  // in 250 for uniform doubles); only then do all passes run.  Three passes less, 6 us.
+  const unsigned long long vary = sm.vary;
+  unsigned long long vary_top      = vary;
+  int lo                        = 0;
+  if constexpr (sizeof(KeyT) == 8) {
+    const int hb = vary ? 63 - __builtin_clzll(vary) : 0;
+    if (hb >= 40) {
+      lo    = 8 * ((hb + 1 - 40 + 7) / 8);
+      vary_top = vary & ~((1ull << lo) - 1);
+    }
+  }
   block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
-                                                   (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, sm.vary);
+                                                   (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, vary_top);
+  if (vary_top != vary) {  // (same in every thread)
+    int bad = 0;
+#pragma unroll
+    for (int j = 0; j < IPT; ++j) {
+      const uint32_t e = (uint32_t)tid * IPT + j;
+      if (e > 0 && e < S) {
+        const unsigned long long a = (unsigned long long)sm.keys[e - 1], b = (unsigned long long)sm.keys[e];
+        bad |= ((a >> lo) == (b >> lo) && a != b) ? 1 : 0;
+      }
+    }
+    if (__syncthreads_or(bad))
+      block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
+                                                       (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, vary);
+  }
   // the sorted sample is still in sm.keys; splitter t = the last sample of stretch t
   KeyT* spl = r.splitters;
   if (p.attempt) {
@@ -837,9 +878,21 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   constexpr int NT = BK_NT, CAP = NT * IPT;
   using PayT = typename std::conditional<PAY == PAY_I64, int64_t, uint32_t>::type;
   constexpr bool HAS_PAY = PAY != PAY_NONE;
-  __shared__ BlockSortSmem<KeyT, PayT, HAS_PAY, NT, IPT> sm;
+  // Keys and payload of a bin side by side in LDS where 16 slots per thread of both fit (8 bytes
+  // in all); else room for 16384 elements of the wider of the two, which holds keys and
+  // payload side by side for bins of up to 8192 elements and one after the other beyond.
+  constexpr int PAYB    = HAS_PAY ? (int)sizeof(PayT) : 0;
+  constexpr bool SHARE  = HAS_PAY && IPT == 16 && (int)sizeof(KeyT) + PAYB > 8;
+  constexpr int WIDER   = (int)sizeof(KeyT) > PAYB ? (int)sizeof(KeyT) : PAYB;
+  constexpr int HALF    = NT * (IPT < 8 ? IPT : 8);  // elements the loop through global memory stages
+  __shared__ uint32_t whist[(NT / 64) * RADIX];
+  __shared__ uint32_t wave_tot[NT / 64];
+  __shared__ __attribute__((aligned(16))) unsigned char store[SHARE ? NT * IPT * WIDER : NT * IPT * ((int)sizeof(KeyT) + PAYB)];
   __shared__ uint32_t gbase[RADIX];
   __shared__ uint32_t tbase[RADIX];
+  KeyT* const skeys = reinterpret_cast<KeyT*>(store);
+  PayT* const spay  = reinterpret_cast<PayT*>(store + (size_t)(SHARE ? HALF : NT * IPT) * sizeof(KeyT));
+  static_assert(!SHARE || (size_t)HALF * (sizeof(KeyT) + sizeof(PayT)) <= sizeof(store), "both halves fit");
   if (p.flags && p.flags[1] == 0) return;  // an attempt that did not go through
   const BucketRow<KeyT, PayT> r(p, blockIdx.y);
   const int tid = threadIdx.x;
@@ -868,8 +921,8 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   const int nbits = diff ? 64 - __builtin_clzll(diff) : 0;
   const int xform = p.keys_travel ? (int)XF_UNSIGNED : p.xform;
   if (len > p.cap) {
-    bucket_sort_long<KeyT, PAY, (IPT < 8 ? IPT : 8)>(p, r, start, len, lo, nbits > 0 ? nbits : 1, xform, sm.whist, sm.wave_tot, sm.keys,
-                                     sm.pay, gbase, tbase);
+    bucket_sort_long<KeyT, PAY, (IPT < 8 ? IPT : 8)>(p, r, start, len, lo, nbits > 0 ? nbits : 1, xform, whist,
+                                                     wave_tot, skeys, spay, gbase, tbase);
     return;
   }
   // The bin in registers, in the instantiation for exactly its number of rows per wavefront:
@@ -888,8 +941,10 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
         if constexpr (HAS_PAY) pv[i] = pbuf[start + e];
       }
     }
-    block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, RR, RR>(sm.whist, sm.wave_tot, sm.keys, sm.pay, el, pv, len, lo,
-                                                           nbits, xform, p.rank_by_add, ~0ull);
+    constexpr bool SHARED_LDS = SHARE && NT * RR > HALF;
+    block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, RR, RR, SHARED_LDS>(
+      whist, wave_tot, skeys, SHARED_LDS ? reinterpret_cast<PayT*>(store) : spay, el, pv, len, lo, nbits, xform,
+      p.rank_by_add, ~0ull);
 #pragma unroll
     for (int i = 0; i < RR; ++i) {
       const uint32_t e = geo.wbase + i * 64;

@@ -346,9 +346,10 @@ struct Plan {
   size_t total = 0;
 };
 
-// Slots per thread of the bin sort (1024 threads): the bin and its payload are staged in LDS
-// between the passes, 128 KB of it.
-constexpr int bucket_sort_ipt(int kb, int pay) { return kb + pay_bytes_of(pay) <= 8 ? 16 : 8; }
+// Slots per thread of the bin sort (1024 threads): the bin is staged in LDS between the
+// passes, 128 KB of it; keys and payload of more than 8 bytes together share that room (side
+// by side up to 8192 elements, one after the other beyond).
+constexpr int bucket_sort_ipt(int, int) { return 16; }
 // The scatter walks tiles of 1024 * 4 elements while that gives every CU a chunk of at most two
 // tiles, and tiles as large as the staging area in LDS allows (element, payload, 2 bytes for the
 // bin) beyond that.

@@ -263,7 +263,7 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *                         their length
  *   bucket_bins           number of bins, 2 .. 256 (0: built in, one per 1024 elements)
  *   bucket_cap            longest bin that is sorted in registers; longer ones take the
- *                         workgroup's loop through global memory (0: built in, 8192 or 16384)
+ *                         workgroup's loop through global memory (0: built in, 16384)
  *   bucket_oversample     sample keys drawn per bin, 1 .. 16 (0: built in, 16; fewer samples give
  *                         uneven bins: tests of bins that outgrow the registers)
  *   low_cardinality       single rows too long for that path, 4- and 8-byte keys, outputs apart

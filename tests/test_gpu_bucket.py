@@ -123,7 +123,8 @@ def test_where_the_path_ends_by_itself(abi):
     assert bucket(np.int32, 1 << 21, 1 << 21, False) and bucket(np.int32, 1 << 21, 1 << 21, True)
     assert not bucket(np.int32, (1 << 21) + 1, (1 << 21) + 1, False)
     assert bucket(np.int32, 3 << 19, 3 << 16, False) and not bucket(np.int32, 1 << 21, 1 << 18, False)
-    assert bucket(np.float64, 1 << 21, 1 << 21, False) and not bucket(np.float64, 1 << 21, 1 << 21, True)
+    assert bucket(np.float64, 1 << 21, 1 << 21, False) and bucket(np.float64, 1 << 21, 1 << 21, True)
+    assert not bucket(np.float64, (1 << 21) + 1, (1 << 21) + 1, True)
     assert bucket(np.int64, 1 << 22, 1 << 19, True) and not bucket(np.int64, 1 << 23, 1 << 19, True)
     assert bucket(np.int16, 1 << 19, 1 << 19, False) and not bucket(np.int16, 1 << 20, 1 << 20, False)
     assert bucket(np.float16, 1 << 20, 1 << 20, False)
@@ -220,6 +221,32 @@ def test_uneven_bins_from_a_thin_sample(abi, dtype):
         a = random_array(dtype, n, rng)
         check(abi, a, options=Options(bucket_oversample=1))
         check(abi, a, options=Options(bucket_oversample=3, bucket_cap=2048))
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.uint64, np.float64], ids=lambda d: np.dtype(d).name)
+def test_sample_keys_that_agree_in_their_upper_bits(abi, dtype):
+    """The sample of 8-byte keys is sorted by the 40 most significant bits that vary, and by all
+    of them only if two sample keys agree in those and differ below: clusters far apart with
+    small differences inside (every sample key has a neighbour like that), clusters next to
+    unique keys, and keys that vary in exactly 40 and 41 bits."""
+    rng = np.random.default_rng(79)
+    n = 200001
+    noise = rng.integers(0, 1 << 20, n)
+    inputs = {}
+    if np.dtype(dtype).kind == "f":
+        inputs["two clusters"] = np.where(rng.integers(0, 2, n) == 0, 1.0, 1e300) * (1.0 + noise * 2.0**-52)
+        inputs["clusters and unique"] = np.where(rng.integers(0, 4, n) == 0, 1.0 + noise * 2.0**-52, rng.standard_normal(n))
+    else:
+        far = np.array([0, 1 << 62, (1 << 62) + (1 << 45)], dtype=np.uint64)
+        inputs["three clusters"] = (far[rng.integers(0, 3, n)] + noise.astype(np.uint64)).astype(dtype)
+        inputs["40 bits"] = rng.integers(0, 1 << 40, n).astype(dtype)
+        inputs["41 bits"] = rng.integers(0, 1 << 41, n).astype(dtype)
+        inputs["clusters and unique"] = np.where(rng.integers(0, 4, n) == 0, noise, rng.integers(0, 1 << 62, n)).astype(dtype)
+    for name, a in inputs.items():
+        a = a.astype(dtype)
+        print(f"bucket upper bits dtype={np.dtype(dtype).name} case={name}", flush=True)
+        assert "strategy=bucket" in abi.describe_plan(dtype, n, n, True)
+        check(abi, a)
 
 
 def test_path_can_be_switched_off_per_call(abi):
