@@ -35,8 +35,9 @@ namespace misort {
 constexpr int BK_SLOTS      = 256;  // splitter table: 255 splitters at most, padded with the largest key
 constexpr int BK_BINS       = 512;
 constexpr int BK_OVERSAMPLE = 16;   // samples per splitter interval
+constexpr int BK_OVERSAMPLE_MAX = 32;  // for rows whose bins average more than 5/12 of what the bin sort holds
 constexpr int BK_PLAN_NT    = 1024;  // the planning workgroup sorts up to 1024 * 4 sample keys
-constexpr int BK_PLAN_IPT   = 4;
+constexpr int BK_PLAN_IPT   = 4;  // 4096 sample keys (8 for the 8192 of BK_OVERSAMPLE_MAX)
 constexpr int BK_COUNT_NT   = 1024;
 constexpr int BK_NT         = 1024;  // scatter and bin sort
 
@@ -51,13 +52,16 @@ struct BucketParams {
   uint32_t* chunk_hist;  // [n_chunks][BK_BINS]
   uint32_t* slab_tot;    // [n_slabs][BK_BINS], cleared by the plan kernel
   uint32_t* bin_start;   // [BK_BINS + 1] first position of every bin, written by chunk 0 of the scatter
+  unsigned long long* chunk_range;  // [n_chunks][2] smallest and largest key of every chunk (count kernel)
+  unsigned long long* key_range;    // [2] smallest and largest key of the row (chunk 0 of the scatter)
   // Several rows of the same length are sorted side by side: the second launch dimension is the
   // row, and every pointer above (but flags) is the first row's: row r has its elements at
   // r * n, its splitters at r * BK_SLOTS, its slab totals at r * n_slabs * BK_BINS, its chunk
-  // counts at r * n_chunks * BK_BINS and its bin starts at r * (BK_BINS + 1).
+  // counts at r * n_chunks * BK_BINS, its bin starts at r * (BK_BINS + 1), its chunks' key ranges
+  // at r * n_chunks * 2 and its own at r * 2.
   uint32_t n;            // elements in a row
   uint32_t n_split;      // splitters in use
-  uint32_t oversample;   // samples per bin (BK_OVERSAMPLE at most)
+  uint32_t oversample;   // samples per bin (BK_OVERSAMPLE_MAX at most)
   uint32_t tile, tiles_per_chunk, n_chunks, chunks_per_slab, n_slabs;
   uint32_t cap;          // longest bin sorted in registers
   int64_t index_offset;
@@ -94,6 +98,8 @@ struct BucketRow {
   uint32_t* slab_tot;
   uint32_t* chunk_hist;
   uint32_t* bin_start;
+  unsigned long long* chunk_range;
+  unsigned long long* key_range;
   __device__ __forceinline__ BucketRow(const BucketParams& p, uint32_t row)
   {
     const size_t e0 = (size_t)row * p.n;
@@ -109,6 +115,8 @@ struct BucketRow {
     slab_tot   = p.slab_tot + (size_t)row * p.n_slabs * BK_BINS;
     chunk_hist = p.chunk_hist + (size_t)row * p.n_chunks * BK_BINS;
     bin_start  = p.bin_start + (size_t)row * (BK_BINS + 1);
+    chunk_range = p.chunk_range + (size_t)row * p.n_chunks * 2;
+    key_range   = p.key_range + (size_t)row * 2;
   }
 };
 
@@ -213,11 +221,16 @@ __device__ __forceinline__ BlockSortGeom block_sort_geom(uint32_t len)
 // lie beyond the elements have no valid lane and do nothing)
 // SHARED_LDS: skeys and spay are the same memory (16384 elements of 12 or 16 bytes do not fit
 // the LDS side by side); the payload then follows the keys through it in a second step.
+// check_lo > 0 (8-byte keys): the caller has left the passes below bit check_lo out of `vary`;
+// the return value says whether this thread saw two neighbours of the result that agree in
+// the bits from check_lo up and differ below, in which case the result is not in order yet
+// and the caller runs all passes (from any order, and stable: equal keys never trade places).
 template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT, int RR, bool SHARED_LDS = false>
-__device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t* wave_tot, KeyT* skeys,
+__device__ __forceinline__ bool block_radix_sort_rows(uint32_t* whist, uint32_t* wave_tot, KeyT* skeys,
                                                       PayT* spay, KeyT (&el)[IPT],
                                                       PayT (&pay)[HAS_PAY ? IPT : 1], uint32_t len, KeyT base,
-                                                      int nbits, int xform, int by_add, unsigned long long vary)
+                                                      int nbits, int xform, int by_add, unsigned long long vary,
+                                                      int check_lo = 0)
 {
   static_assert(NT % RADIX == 0 && RR <= IPT, "whole groups of one thread per digit value");
   constexpr int NW  = NT / 64;
@@ -233,6 +246,13 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
   const bool is_float  = xform == XF_FLOAT;
   const KeyT flip      = xform == XF_SIGNED ? (KeyT)((KeyT)1 << (sizeof(KeyT) * 8 - 1)) : (KeyT)0;
   for (int i = tid; i < NW * RADIX; i += NT) whist[i] = 0;  // (a pass leaves them cleared for the next)
+  int last_shift = -1;
+  bool bad       = false;
+  if constexpr (sizeof(KeyT) == 8) {
+    if (check_lo)
+      for (int sh = 0; sh < nbits; sh += RADIX_BITS)
+        if ((vary >> sh) & (RADIX - 1)) last_shift = sh;
+  }
   for (int shift = 0; shift < nbits; shift += RADIX_BITS) {
     if (((vary >> shift) & (RADIX - 1)) == 0) continue;  // (same in every thread)
     uint32_t d[RR], r[RR];
@@ -289,6 +309,20 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
         if constexpr (HAS_PAY && !SHARED_LDS) pay[i] = spay[wbase + i * 64];
       }
     }
+    if constexpr (sizeof(KeyT) == 8) {
+      if (shift == last_shift) {  // (only with check_lo, in the last pass that runs)
+#pragma unroll
+        for (int i = 0; i < RR; ++i) {
+          const uint32_t e = wbase + i * 64;
+          if (e > 0 && e < len) {
+            const KeyT pe = skeys[e - 1];
+            const KeyT ka = (KeyT)((is_float ? float_to_key(pe) : (KeyT)(pe ^ flip)) - base);
+            const KeyT kb = (KeyT)((is_float ? float_to_key(el[i]) : (KeyT)(el[i] ^ flip)) - base);
+            bad |= (ka >> check_lo) == (kb >> check_lo) && ka != kb;
+          }
+        }
+      }
+    }
     if constexpr (HAS_PAY && SHARED_LDS) {
       __syncthreads();  // (every key has been read back)
 #pragma unroll
@@ -301,21 +335,23 @@ __device__ __forceinline__ void block_radix_sort_rows(uint32_t* whist, uint32_t*
       // (the next pass writes keys only after two more barriers)
     }
   }
+  return bad;
 }
 
 // xform: XF_UNSIGNED, XF_SIGNED or XF_FLOAT (complex keys are transformed before they get here)
 template <typename KeyT, typename PayT, bool HAS_PAY, int NT, int IPT>
-__device__ __forceinline__ void block_radix_sort(uint32_t* whist /* (NT / 64) * RADIX */,
+__device__ __forceinline__ bool block_radix_sort(uint32_t* whist /* (NT / 64) * RADIX */,
                                                  uint32_t* wave_tot /* NT / 64 */,
                                                  KeyT* skeys /* NT * IPT */, PayT* spay /* NT * IPT */,
                                                  KeyT (&el)[IPT], PayT (&pay)[HAS_PAY ? IPT : 1],
                                                  uint32_t len, KeyT base, int nbits, int xform, int by_add,
-                                                 unsigned long long vary = ~0ull /* bits in which keys differ */)
+                                                 unsigned long long vary = ~0ull /* bits in which keys differ */,
+                                                 int check_lo = 0)
 {
   const uint32_t R = block_sort_geom<NT>(len).R;
-#define MISORT_BK_ROWS(RR)                                                                                   \
-  block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, IPT, RR>(whist, wave_tot, skeys, spay, el, pay, len, base, \
-                                                          nbits, xform, by_add, vary)
+#define MISORT_BK_ROWS(RR)                                                                                          \
+  return block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, IPT, RR>(whist, wave_tot, skeys, spay, el, pay, len, base, \
+                                                                 nbits, xform, by_add, vary, check_lo)
   if (R == 1) MISORT_BK_ROWS(1);
   else if (R == 2) MISORT_BK_ROWS(2);
   else if (R == 4) MISORT_BK_ROWS(4);
@@ -324,15 +360,30 @@ __device__ __forceinline__ void block_radix_sort(uint32_t* whist /* (NT / 64) * 
     else if constexpr (IPT >= 16) MISORT_BK_ROWS(16);
   }
 #undef MISORT_BK_ROWS
+  return false;
+}
+
+// The bits that 8-byte keys are sorted by first: the 40 or more most significant of those that
+// can differ, from a digit boundary up (`vary`; bits [0, nbits) of key - base).  Two of 4096 or 16384 keys that agree in all
+// of them and differ below are rare (uniform doubles: one sample in 250), so the passes
+// below mostly never run.  Returns the first bit kept (0: all passes run anyway).
+__device__ __forceinline__ int upper_bits_first(unsigned long long vary, unsigned long long& vary_top)
+{
+  vary_top     = vary;
+  const int hb = vary ? 63 - __builtin_clzll(vary) : 0;
+  if (hb < 40) return 0;
+  const int lo = 8 * ((hb + 1 - 40) / 8);  // (40 to 47 bits stay)
+  vary_top     = vary & ~((1ull << lo) - 1);
+  return vary_top != vary ? lo : 0;
 }
 
 // ---------------------------------------------------------------------------------------
 // plan: splitters from a sorted sample; also clears the slab totals of the count kernel
 // ---------------------------------------------------------------------------------------
-template <typename KeyT>
+template <typename KeyT, int IPT = BK_PLAN_IPT>
 __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
 {
-  constexpr int NT = BK_PLAN_NT, IPT = BK_PLAN_IPT;
+  constexpr int NT = BK_PLAN_NT;
   __shared__ BlockSortSmem<KeyT, uint32_t, false, NT, IPT> sm;
   const int tid = threadIdx.x;
   const BucketRow<KeyT, uint32_t> r(p, blockIdx.x);  // one workgroup per row (the payload is not touched)
@@ -380,36 +431,17 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
     if ((tid & 63) == 0 && vv) atomicOr(&sm.vary, vv);
     __syncthreads();
   }
-  // 8-byte keys that vary in more than 40 bits: the passes over the 40 most significant of
-  // those bits put the sample in order unless two sample keys agree in all of them and differ
-  // below (for 4096 keys drawn from doubles or 64-bit integers a rare event: about one sample
-  // in 250 for uniform doubles); only then do all passes run.  Three passes less, 6 us.
-  const unsigned long long vary = sm.vary;
-  unsigned long long vary_top      = vary;
-  int lo                        = 0;
-  if constexpr (sizeof(KeyT) == 8) {
-    const int hb = vary ? 63 - __builtin_clzll(vary) : 0;
-    if (hb >= 40) {
-      lo    = 8 * ((hb + 1 - 40 + 7) / 8);
-      vary_top = vary & ~((1ull << lo) - 1);
-    }
-  }
-  block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
-                                                   (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, vary_top);
-  if (vary_top != vary) {  // (same in every thread)
-    int bad = 0;
-#pragma unroll
-    for (int j = 0; j < IPT; ++j) {
-      const uint32_t e = (uint32_t)tid * IPT + j;
-      if (e > 0 && e < S) {
-        const unsigned long long a = (unsigned long long)sm.keys[e - 1], b = (unsigned long long)sm.keys[e];
-        bad |= ((a >> lo) == (b >> lo) && a != b) ? 1 : 0;
-      }
-    }
-    if (__syncthreads_or(bad))
-      block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
-                                                       (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, vary);
-  }
+  // (8-byte keys: by the upper 40 varying bits first, by all of them only if that left two
+  // sample keys in the wrong order: three passes less, 3-6 us)
+  unsigned long long vary_top = sm.vary;
+  int lo                      = 0;
+  if constexpr (sizeof(KeyT) == 8) lo = upper_bits_first(sm.vary, vary_top);
+  const bool bad = block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay,
+                                                                   S, (KeyT)0, (int)sizeof(KeyT) * 8, XF_UNSIGNED,
+                                                                   p.rank_by_add, vary_top, lo);
+  if (lo && __syncthreads_or(bad ? 1 : 0))  // (lo is the same in every thread)
+    block_radix_sort<KeyT, uint32_t, false, NT, IPT>(sm.whist, sm.wave_tot, sm.keys, sm.pay, k, nopay, S, (KeyT)0,
+                                                     (int)sizeof(KeyT) * 8, XF_UNSIGNED, p.rank_by_add, sm.vary);
   // the sorted sample is still in sm.keys; splitter t = the last sample of stretch t
   KeyT* spl = r.splitters;
   if (p.attempt) {
@@ -455,7 +487,7 @@ __global__ void __launch_bounds__(BK_PLAN_NT) bucket_plan_kernel(BucketParams p)
 // ---------------------------------------------------------------------------------------
 // count: keys per bin of every chunk, added up per slab of chunks
 // ---------------------------------------------------------------------------------------
-template <typename KeyT>
+template <typename KeyT, bool TRACK = true>
 __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams p)
 {
   constexpr int NT = BK_COUNT_NT, NW = NT / 64;
@@ -464,6 +496,7 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
   if (p.flags && p.flags[0] == 0) return;  // an attempt that the plan kernel called off
   const BucketRow<KeyT, uint32_t> r(p, blockIdx.y);
   const int tid = threadIdx.x, wave = tid >> 6;
+  __shared__ unsigned long long wmin[NW], wmax[NW];
   for (int i = tid; i < NW * BK_BINS; i += NT) hist[i] = 0;
   load_splitters<KeyT, NT>(tab, r.splitters);
   const uint32_t chunk = blockIdx.x;
@@ -482,10 +515,24 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
       raw[u]           = in[i < b1 ? i : b0];
     }
   };
+  // (the smallest and the largest key of the chunk as well: the first and the last bin have no
+  // splitter on their outer side, and the bin sort takes its bits from the bounds of a bin;
+  // a lane past the end holds the chunk's first key again)
+  // (not on a long row's attempt, whose bins that need sorting are few and short: the bounds
+  // are then the smallest and the largest key there is)
+  // (TRACK = false: a compare more per key in this loop cost the count of 2^28 keys 0.16 ms)
+  KeyT kmin = TRACK ? KeyOps<KeyT>::max_key() : (KeyT)0, kmax = TRACK ? (KeyT)0 : KeyOps<KeyT>::max_key();
   auto consume = [&](const KeyT (&raw)[U], uint64_t i0) {
     uint32_t b[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) b[u] = bin_of(tab, KeyOps<KeyT>::to_key(raw[u], p.xform));
+    for (int u = 0; u < U; ++u) {
+      const KeyT k = KeyOps<KeyT>::to_key(raw[u], p.xform);
+      if constexpr (TRACK) {
+        kmin = k < kmin ? k : kmin;
+        kmax = k > kmax ? k : kmax;
+      }
+      b[u] = bin_of(tab, k);
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (i0 + (uint64_t)u * NT + tid < b1) atomicAdd(&my[b[u]], 1u);
@@ -504,7 +551,34 @@ __global__ void __launch_bounds__(BK_COUNT_NT) bucket_count_kernel(BucketParams 
       i0 = i2;
     }
   }
+  {
+    unsigned long long mn = (unsigned long long)kmin, mx = (unsigned long long)kmax;
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) {
+      const unsigned long long a = __shfl_xor(mn, sft, 64), b = __shfl_xor(mx, sft, 64);
+      mn = a < mn ? a : mn;
+      mx = b > mx ? b : mx;
+    }
+    if ((tid & 63) == 0) {
+      wmin[wave] = mn;
+      wmax[wave] = mx;
+    }
+  }
   __syncthreads();
+  if (tid < 64) {  // (one wavefront: the NW partial results in its first lanes)
+    static_assert(NW <= 64 && (NW & (NW - 1)) == 0, "a power of two of partial results");
+    unsigned long long mn = wmin[tid & (NW - 1)], mx = wmax[tid & (NW - 1)];
+#pragma unroll
+    for (int sft = NW / 2; sft > 0; sft >>= 1) {
+      const unsigned long long a = __shfl_xor(mn, sft, 64), b = __shfl_xor(mx, sft, 64);
+      mn = a < mn ? a : mn;
+      mx = b > mx ? b : mx;
+    }
+    if (tid == 0) {
+      r.chunk_range[2 * chunk]     = mn;
+      r.chunk_range[2 * chunk + 1] = mx;
+    }
+  }
   uint32_t* out  = r.chunk_hist + (uint64_t)chunk * BK_BINS;
   uint32_t* slab = r.slab_tot + (uint64_t)(chunk / p.chunks_per_slab) * BK_BINS;
   for (int b = tid; b < BK_BINS; b += NT) {
@@ -561,11 +635,32 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
     }
   };
   if (tile0 < tile_end) load_tile(tile0);
+  __shared__ unsigned long long wmin[NW], wmax[NW];  // chunk 0: the row's smallest and largest key
   load_splitters<KeyT, NT>(tab, r.splitters);
 
   // ---- where this chunk's elements of every bin start: the bins before (all chunks), the
   // same bin in the slabs before this chunk's and in the chunks before it inside its slab
   {
+    // chunk 0 also works out the row's smallest and largest key from the chunks', for the bin
+    // sort of the first and the last bin
+    if (chunk == 0) {
+      unsigned long long mn = ~0ull, mx = 0ull;
+      for (uint32_t c = tid; c < p.n_chunks; c += NT) {
+        const unsigned long long a = r.chunk_range[2 * c], b = r.chunk_range[2 * c + 1];
+        mn = a < mn ? a : mn;
+        mx = b > mx ? b : mx;
+      }
+#pragma unroll
+      for (int sft = 32; sft > 0; sft >>= 1) {
+        const unsigned long long a = __shfl_xor(mn, sft, 64), b = __shfl_xor(mx, sft, 64);
+        mn = a < mn ? a : mn;
+        mx = b > mx ? b : mx;
+      }
+      if (lane == 0) {
+        wmin[wave] = mn;
+        wmax[wave] = mx;
+      }
+    }
     // (the first half of the workgroup adds up the slabs, the second the chunks before this
     // one in its slab, four loads in flight each: one after the other the up to 30 reads were
     // a third of the kernel's time on short rows)
@@ -626,6 +721,15 @@ __global__ void __launch_bounds__(BK_NT) bucket_scatter_kernel(BucketParams p)
       if (chunk == 0) {
         r.bin_start[tid] = start;
         if (tid == BK_BINS - 1) r.bin_start[BK_BINS] = p.n;
+        if (tid == 0) {  // (the wavefronts' results are in place since the barrier above)
+          unsigned long long mn = wmin[0], mx = wmax[0];
+          for (int w = 1; w < NW; ++w) {
+            mn = wmin[w] < mn ? wmin[w] : mn;
+            mx = wmax[w] > mx ? wmax[w] : mx;
+          }
+          r.key_range[0] = mn;
+          r.key_range[1] = mx;
+        }
       }
     }
     __syncthreads();
@@ -914,9 +1018,12 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
   if (len == 0) return;
   // the keys of the bin lie strictly between the splitters lo and hi: sorted by key - lo, which
   // is below hi - lo and so has that many bits at most
+  // (the first bin starts at the row's smallest key, and no bin reaches beyond its largest:
+  // the last one would else sort every bit up to the largest key there is)
   const KeyT* spl = r.splitters;
-  const KeyT lo   = g > 0 ? spl[g - 1] : (KeyT)0;
-  const KeyT hi   = spl[g];
+  const KeyT kmax = (KeyT)r.key_range[1];
+  const KeyT lo   = g > 0 ? spl[g - 1] : (KeyT)r.key_range[0];
+  const KeyT hi   = spl[g] < kmax ? spl[g] : kmax;
   const unsigned long long diff = (unsigned long long)(KeyT)(hi - lo);
   const int nbits = diff ? 64 - __builtin_clzll(diff) : 0;
   const int xform = p.keys_travel ? (int)XF_UNSIGNED : p.xform;
@@ -942,9 +1049,17 @@ __global__ void __launch_bounds__(BK_NT) bucket_sort_kernel(BucketParams p)
       }
     }
     constexpr bool SHARED_LDS = SHARE && NT * RR > HALF;
-    block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, RR, RR, SHARED_LDS>(
-      whist, wave_tot, skeys, SHARED_LDS ? reinterpret_cast<PayT*>(store) : spay, el, pv, len, lo, nbits, xform,
-      p.rank_by_add, ~0ull);
+    unsigned long long bits = nbits >= 64 ? ~0ull : (1ull << nbits) - 1;  // key - lo lies below 2^nbits
+    int first_bit           = 0;
+    if constexpr (sizeof(KeyT) == 8) first_bit = upper_bits_first(bits, bits);
+    for (;;) {
+      const bool bad = block_radix_sort_rows<KeyT, PayT, HAS_PAY, NT, RR, RR, SHARED_LDS>(
+        whist, wave_tot, skeys, SHARED_LDS ? reinterpret_cast<PayT*>(store) : spay, el, pv, len, lo, nbits, xform,
+        p.rank_by_add, bits, first_bit);
+      if (first_bit == 0 || !__syncthreads_or(bad ? 1 : 0)) break;  // (first_bit is the same in every thread)
+      first_bit = 0;
+      bits      = ~0ull;
+    }
 #pragma unroll
     for (int i = 0; i < RR; ++i) {
       const uint32_t e = geo.wbase + i * 64;

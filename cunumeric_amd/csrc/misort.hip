@@ -138,7 +138,7 @@ struct PlanOptions {
   int bucket_path = -1;                 // < 0: the built-in choice; 0: never; > 0: wherever it is able to run
   unsigned bucket_bins = 0;             // 0: the built-in choice; else splitter intervals, 2 .. 256
   unsigned bucket_cap = 0;              // 0: the built-in choice; else the longest bin sorted in registers
-  unsigned bucket_oversample = 0;       // 0: the built-in choice; else samples per bin, 1 .. 16
+  unsigned bucket_oversample = 0;       // 0: the built-in choice; else samples per bin, 1 .. 32
   int low_cardinality = -1;             // long rows try the four-launch path first: < 0: rows of 2^27 elements
                                         // and more, where the sample holds few distinct keys; 0: never;
                                         // 1: the same for every length; 2: with any sample
@@ -339,6 +339,7 @@ struct Plan {
   uint32_t bk_split = 0, bk_cap = 0, bk_tile = 0, bk_tiles_per_chunk = 0, bk_chunks = 0, bk_slabs = 0;
   uint32_t bk_oversample = BK_OVERSAMPLE;
   size_t off_bk_splitters = 0, off_bk_slab_tot = 0, off_bk_chunk_hist = 0, off_bk_bin_start = 0;
+  size_t off_bk_chunk_range = 0, off_bk_key_range = 0;
   // radix plans of one long row: the four-launch path is tried first, and goes through where
   // the keys take few distinct values (1: if the sample says so; 2: tried with any sample)
   int low_card = 0;
@@ -472,7 +473,13 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
       pl.strategy = S_BUCKET;
       pl.bk_split = (uint32_t)bins - 1;
       pl.bk_cap   = (uint32_t)cap;
-      if (opt.bucket_oversample >= 1 && opt.bucket_oversample <= (unsigned)BK_OVERSAMPLE)
+      // 16 samples per bin: a bin of twice the average is a 7e-4 event per bin, one of three
+      // times 1e-8.  Rows whose bins average more than 5/12 of the capacity (2.4 times the
+      // average fills a bin: 1.5e-5) draw 32 (twice the average: 4e-6), or one sort in six at the
+      // longest rows would find a bin that takes the loop through global memory; that costs the
+      // plan kernel 8 us more.
+      if (pl.row_len > bins * (cap * 5 / 12)) pl.bk_oversample = BK_OVERSAMPLE_MAX;
+      if (opt.bucket_oversample >= 1 && opt.bucket_oversample <= (unsigned)BK_OVERSAMPLE_MAX)
         pl.bk_oversample = opt.bucket_oversample;
     }
   }
@@ -497,6 +504,8 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
     pl.off_bk_slab_tot    = take(pl.rows * pl.bk_slabs * BK_BINS * sizeof(uint32_t));
     pl.off_bk_chunk_hist  = take(pl.rows * pl.bk_chunks * BK_BINS * sizeof(uint32_t));
     pl.off_bk_bin_start   = take(pl.rows * (BK_BINS + 1) * sizeof(uint32_t));
+    pl.off_bk_chunk_range = take(pl.rows * pl.bk_chunks * 2 * sizeof(unsigned long long));
+    pl.off_bk_key_range   = take(pl.rows * 2 * sizeof(unsigned long long));
     pl.off_bk_flags       = take(2 * sizeof(uint32_t));
   };
 
@@ -958,6 +967,8 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int 
   p.slab_tot        = reinterpret_cast<uint32_t*>(S + pl.off_bk_slab_tot);
   p.chunk_hist      = reinterpret_cast<uint32_t*>(S + pl.off_bk_chunk_hist);
   p.bin_start       = reinterpret_cast<uint32_t*>(S + pl.off_bk_bin_start);
+  p.chunk_range     = reinterpret_cast<unsigned long long*>(S + pl.off_bk_chunk_range);
+  p.key_range       = reinterpret_cast<unsigned long long*>(S + pl.off_bk_key_range);
   p.n               = (uint32_t)pl.row_len;
   p.n_split         = pl.bk_split;
   p.oversample      = pl.bk_oversample;
@@ -976,10 +987,16 @@ static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int 
   constexpr int IPT = bucket_sort_ipt(sizeof(KeyT), PAY);
   const unsigned rows = (unsigned)pl.rows;
   L.run(K_BUCKET_PLAN, [&] {
-    hipLaunchKernelGGL((bucket_plan_kernel<KeyT>), dim3(rows), dim3(BK_PLAN_NT), 0, L.stream, p);
+    if ((pl.bk_split + 1) * pl.bk_oversample <= (uint32_t)BK_PLAN_NT * BK_PLAN_IPT)
+      hipLaunchKernelGGL((bucket_plan_kernel<KeyT, BK_PLAN_IPT>), dim3(rows), dim3(BK_PLAN_NT), 0, L.stream, p);
+    else
+      hipLaunchKernelGGL((bucket_plan_kernel<KeyT, 2 * BK_PLAN_IPT>), dim3(rows), dim3(BK_PLAN_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_COUNT, [&] {
-    hipLaunchKernelGGL((bucket_count_kernel<KeyT>), dim3(pl.bk_chunks, rows), dim3(BK_COUNT_NT), 0, L.stream, p);
+    if (attempt)
+      hipLaunchKernelGGL((bucket_count_kernel<KeyT, false>), dim3(pl.bk_chunks, rows), dim3(BK_COUNT_NT), 0, L.stream, p);
+    else
+      hipLaunchKernelGGL((bucket_count_kernel<KeyT, true>), dim3(pl.bk_chunks, rows), dim3(BK_COUNT_NT), 0, L.stream, p);
   });
   L.run(K_BUCKET_SCATTER, [&] {
     constexpr int LARGE = bucket_scatter_ipt_large(sizeof(KeyT), PAY);

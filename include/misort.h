@@ -264,8 +264,9 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *   bucket_bins           number of bins, 2 .. 256 (0: built in, one per 1024 elements)
  *   bucket_cap            longest bin that is sorted in registers; longer ones take the
  *                         workgroup's loop through global memory (0: built in, 16384)
- *   bucket_oversample     sample keys drawn per bin, 1 .. 16 (0: built in, 16; fewer samples give
- *                         uneven bins: tests of bins that outgrow the registers)
+ *   bucket_oversample     sample keys drawn per bin, 1 .. 32 (0: built in: 16, and 32 for rows
+ *                         whose bins average more than 5/12 of bucket_cap; fewer samples
+ *                         give uneven bins: tests of bins that outgrow the registers)
  *   low_cardinality       single rows too long for that path, 4- and 8-byte keys, outputs apart
  *                         from the inputs: the path is tried all the same where a sample of the
  *                         row holds at most 255 distinct keys (each of them then gets a bin of
