@@ -52,12 +52,35 @@ def splitters_of(keys: np.ndarray, n_split: int) -> np.ndarray:
     return spl
 
 
-def bin_bits(spl: np.ndarray, g: int):
+def bin_bits(spl: np.ndarray, g: int, kmin: int = 0, kmax: int | None = None):
     """bucket_sort_kernel: keys strictly between splitters g-1 and g are sorted by key - lo,
-    which has at most as many bits as hi - lo."""
-    lo = int(spl[g - 1]) if g > 0 else 0
-    hi = int(spl[g])
+    which has at most as many bits as hi - lo; the first bin starts at the row's smallest key
+    and no bin reaches beyond its largest (count kernel -> chunk 0 of the scatter)."""
+    lo = int(spl[g - 1]) if g > 0 else int(kmin)
+    hi = int(spl[g]) if kmax is None else min(int(spl[g]), int(kmax))
     return lo, (hi - lo).bit_length()
+
+
+def upper_bits_first(nbits: int) -> int:
+    """8-byte keys: the first bit of the 40 to 47 upper ones of [0, nbits) that the bin sort
+    looks at first (0: all of them anyway)."""
+    hb = nbits - 1
+    if hb < 40:
+        return 0
+    return 8 * ((hb + 1 - 40) // 8)
+
+
+def sort_bin(sub: np.ndarray, nbits: int, eight_byte: bool) -> np.ndarray:
+    """Order of a bin by its reduced keys the way block_radix_sort_rows gets there: by the upper
+    bits first; if two neighbours of that order agree in them and differ below, by all bits
+    from that order on (stable passes: equal keys never trade places)."""
+    lo = upper_bits_first(nbits) if eight_byte else 0
+    if lo == 0:
+        return np.argsort(sub, kind="stable")
+    first = np.argsort(sub >> np.uint64(lo), kind="stable")
+    s = sub[first]
+    bad = np.any(((s[1:] >> np.uint64(lo)) == (s[:-1] >> np.uint64(lo))) & (s[1:] != s[:-1]))
+    return first[np.argsort(s, kind="stable")] if bad else first
 
 
 def bucket_argsort(keys: np.ndarray, n_split: int, tile: int = 4096, chunks_per_slab: int = 16):
@@ -104,10 +127,12 @@ def bucket_argsort(keys: np.ndarray, n_split: int, tile: int = 4096, chunks_per_
         s, e = bin_start[2 * g], bin_start[2 * g + 1]
         if e - s < 2:
             continue
-        lo, nbits = bin_bits(spl, g)
+        lo, nbits = bin_bits(spl, g, keys.min(), keys.max())
         idx = scattered[s:e]
-        sub = (keys[idx].astype(np.uint64) - np.uint64(lo)) & np.uint64((1 << nbits) - 1 if nbits < 64 else 0xFFFFFFFFFFFFFFFF)
-        out[s:e] = idx[np.argsort(sub, kind="stable")]
+        full = keys[idx].astype(np.uint64) - np.uint64(lo)
+        sub = full & np.uint64((1 << nbits) - 1 if nbits < 64 else 0xFFFFFFFFFFFFFFFF)
+        assert np.array_equal(sub, full)  # (no key of the bin has a bit beyond nbits)
+        out[s:e] = idx[sort_bin(sub, nbits, keys.dtype.itemsize == 8)]
     for g in range(SLOTS):  # a bin of equal keys holds equal keys
         s, e = bin_start[2 * g + 1], bin_start[2 * g + 2]
         assert e == s or np.all(keys[scattered[s:e]] == keys[scattered[s]])

@@ -36,7 +36,7 @@ def test_sample_places_stay_inside_their_stretch():
 
 
 @pytest.mark.parametrize("case", ["uniform32", "uniform64", "small_range", "two_values", "constant", "sorted",
-                                  "sawtooth", "skewed", "top_keys", "u8", "u16"])
+                                  "sawtooth", "skewed", "top_keys", "u8", "u16", "clusters64", "low_bits64"])
 def test_twin_sorts_like_a_stable_argsort(case):
     rng = np.random.default_rng(hash(case) % 1000)
     n = 50021
@@ -59,6 +59,12 @@ def test_twin_sorts_like_a_stable_argsort(case):
     elif case == "top_keys":
         k = np.where(rng.random(n) < 0.3, np.uint32(0xFFFFFFFF), rng.integers(0, 2**32, n, dtype=np.uint32))
         k = k.astype(np.uint32)
+    elif case == "clusters64":   # neighbours that agree in the upper bits and differ below: all passes
+        far = np.array([0, 1 << 62, (1 << 62) + (1 << 45)], dtype=np.uint64)
+        k = far[rng.integers(0, 3, n)] + rng.integers(0, 1 << 20, n, dtype=np.uint64)
+    elif case == "low_bits64":   # a few huge keys stretch the bins' bounds; the rest differs low down
+        k = rng.integers(0, 1 << 12, n, dtype=np.uint64)
+        k[rng.integers(0, n, 40)] = rng.integers(1 << 50, 1 << 63, 40, dtype=np.uint64)
     elif case == "u8":
         k = rng.integers(0, 256, n, dtype=np.uint8)
     else:
@@ -66,3 +72,12 @@ def test_twin_sorts_like_a_stable_argsort(case):
     for n_split in (1, 12, 48, 255):
         order, bins = tw.bucket_argsort(k, n_split)
         assert np.array_equal(order, np.argsort(k, kind="stable")), (case, n_split)
+
+
+def test_upper_bits_first_rule():
+    assert [tw.upper_bits_first(b) for b in (1, 40, 41, 47, 48, 55, 56, 57, 64)] == [0, 0, 0, 0, 8, 8, 16, 16, 24]
+    rng = np.random.default_rng(3)
+    sub = rng.integers(0, 1 << 20, 5000, dtype=np.uint64) + (rng.integers(0, 2, 5000, dtype=np.uint64) << np.uint64(60))
+    assert np.array_equal(tw.sort_bin(sub, 61, True), np.argsort(sub, kind="stable"))   # falls back to all bits
+    sub = rng.integers(0, 1 << 61, 5000, dtype=np.uint64)
+    assert np.array_equal(tw.sort_bin(sub, 61, True), np.argsort(sub, kind="stable"))   # upper bits suffice
