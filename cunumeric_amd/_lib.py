@@ -62,12 +62,12 @@ class Options(ctypes.Structure):
 
     _fields_ = [("target_chunks", c_size_t), ("early_last_min_bytes", ctypes.c_longlong),
                 ("bucket_path", c_int), ("bucket_bins", ctypes.c_uint), ("bucket_cap", ctypes.c_uint),
-                ("low_cardinality", c_int), ("bucket_oversample", ctypes.c_uint), ("counting_sort", c_int)]
+                ("low_cardinality", c_int), ("bucket_oversample", ctypes.c_uint), ("counting_sort", c_int), ("upper_first", c_int)]
 
     def __init__(self, target_chunks=0, early_last_min_bytes=-1, bucket_path=-1, bucket_bins=0, bucket_cap=0,
-                 low_cardinality=-1, bucket_oversample=0, counting_sort=-1):
+                 low_cardinality=-1, bucket_oversample=0, counting_sort=-1, upper_first=-1):
         super().__init__(target_chunks, early_last_min_bytes, bucket_path, bucket_bins, bucket_cap, low_cardinality,
-                         bucket_oversample, counting_sort)
+                         bucket_oversample, counting_sort, upper_first)
 
 
 class MisortLibraryError(RuntimeError):

@@ -25,6 +25,7 @@
 #include "unique.hpp"
 #include "selftest.hpp"
 #include "bucket.hpp"
+#include "upperfirst.hpp"
 
 namespace misort {
 
@@ -144,6 +145,8 @@ struct PlanOptions {
                                         // 1: the same for every length; 2: with any sample
   int counting_sort = -1;               // one row of 2-byte values: < 0: counted from the built-in length on;
                                         // 0: never; > 0: whenever the row is too long for the row kernels
+  int upper_first = -1;                 // 8-byte keys by their upper 40 bits first (upperfirst.hpp): < 0: from
+                                        // 2^25 elements on; 0: never; 1: any length; 2: whatever the sample says
 };
 
 static int fail(int code, const std::string& msg)
@@ -188,6 +191,8 @@ enum KernelId : int {
   K_BUCKET_COUNT,
   K_BUCKET_SCATTER,
   K_BUCKET_SORT,
+  K_UF_PLAN,
+  K_UF_FIXUP,
   K_NUM
 };
 
@@ -201,7 +206,7 @@ static const char* const kKernelNames[K_NUM] = {
   "count8_fill",     "select_init",     "select_hist",      "select_pick",
   "select_counts",   "select_above",    "select_emit",    "select_split",
   "colsort_wave",    "bucket_plan",     "bucket_count",     "bucket_scatter",
-  "bucket_sort"};
+  "bucket_sort",     "upper_first_plan", "upper_first_fixup"};
 
 // ---------------------------------------------------------------------------------------
 // dtype table
@@ -344,6 +349,10 @@ struct Plan {
   // the keys take few distinct values (1: if the sample says so; 2: tried with any sample)
   int low_card = 0;
   size_t off_bk_flags = 0;
+  // radix plans of 8-byte keys: sorted by the upper five digits first (1: if the sample agrees;
+  // 2: whatever it says), the lower three only if the fix-up finds runs too long to sort
+  int upper_first = 0;
+  size_t off_uf_flags = 0, off_uf_keys = 0;
   size_t total = 0;
 };
 
@@ -609,6 +618,17 @@ static int make_plan(int dtype, size_t volume, size_t sort_dim_size, bool argsor
       pl.bk_cap   = (uint32_t)(BK_NT * bucket_sort_ipt(pl.dt.bytes, pl.pay));
       bucket_tables(kBucketMaxChunksLong);
     }
+    // Long sorts of 8-byte keys: by the upper five digits first, the lower three only if the
+    // fix-up meets runs too long to sort (upperfirst.hpp): five passes and a read of the
+    // result instead of eight passes.  From 2^25 elements on, where the 17 launches of the
+    // eight-pass sort that return at once (0.1 ms) are a few per cent of what is saved; not in
+    // place (the eight-pass sort needs the input again), which the launch sequence checks.
+    if (pl.dt.bytes == 8 && pl.n_passes == 8 && !pl.gather_values && opt.upper_first != 0 &&
+        opt.target_chunks == 0 && (opt.upper_first > 0 || pl.volume >= ((size_t)1 << 25))) {
+      pl.upper_first  = opt.upper_first == 2 ? 2 : 1;
+      pl.off_uf_flags = take(2 * sizeof(uint32_t));
+      if (pl.pay != PAY_NONE) pl.off_uf_keys = take(pl.volume * pl.dt.bytes);  // the result's keys, for the fix-up
+    }
   } else if (pl.strategy == S_COUNT16) {
     // one histogram workgroup per CU and half of the key range, a few rounds of them
     constexpr size_t gran = (size_t)(C16_HIST_NT / 64) * 64 * 8;  // whole 16-byte loads per wavefront
@@ -739,8 +759,66 @@ static void launch_zero(Launcher& L, void* p, size_t bytes)
 template <typename KeyT, int PAY>
 static void bucket_sort_row(Launcher& L, const Plan& pl, const SortArgs& a, int attempt = 0);
 
+// What distinguishes the runs of the pass sequence below: the plain sort (digit_base 0, all
+// digits), and the sort by the upper digits that upperfirst.hpp tries first.
+struct RadixRun {
+  int digit_base            = 0;        // the first pass's digit
+  const uint32_t* done_flag = nullptr;  // the kernels return at once if the word is set
+  const uint32_t* go_flag   = nullptr;  // ... or if this one is clear
+  void* keys_for_fixup      = nullptr;  // where the last pass puts the keys if the caller wants none
+  bool upper_first          = false;
+};
+
+template <typename KeyT, int PAY>
+static void radix_sort_passes(Launcher& L, const Plan& plan, const SortArgs& a, const RadixRun& run);
+
 template <typename KeyT, int PAY>
 static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
+{
+  char* S = a.scratch;
+  // few distinct keys: the four-launch path writes the result, and the kernels below return at once
+  const uint32_t* done_flag = nullptr;
+  const bool outputs_apart  = (a.values_out == nullptr || a.values_out != a.values_in) &&
+                             (a.indices_out == nullptr || a.indices_out != a.indices_in);
+  if constexpr (sizeof(KeyT) == 4 || sizeof(KeyT) == 8) {
+    if (plan.low_card && outputs_apart) {
+      bucket_sort_row<KeyT, PAY>(L, plan, a, plan.low_card);
+      done_flag = reinterpret_cast<const uint32_t*>(S + plan.off_bk_flags) + 1;
+    }
+  }
+  if constexpr (sizeof(KeyT) == 8) {
+    if (plan.upper_first && outputs_apart) {
+      uint32_t* flags = reinterpret_cast<uint32_t*>(S + plan.off_uf_flags);
+      UpperFirstParams up{};
+      up.keys_in     = a.values_in;
+      up.volume      = plan.volume;
+      up.row_len     = plan.row_len;
+      up.xform       = plan.dt.xform;
+      up.low_bits    = RADIX_BITS * upper_first_digit0(plan.dt.xform);
+      up.mode        = plan.upper_first;
+      up.rank_by_add = rank_by_add_on_current_device();
+      up.flags       = flags;
+      up.prior_done  = done_flag;
+      L.run(K_UF_PLAN, [&] {
+        hipLaunchKernelGGL((upper_first_plan_kernel<KeyT>), dim3(1), dim3(UF_PLAN_NT), 0, L.stream, up);
+      });
+      RadixRun first;
+      first.digit_base  = upper_first_digit0(plan.dt.xform);
+      first.go_flag     = flags;
+      first.upper_first = true;
+      const bool caller_keys = !plan.argsort || a.values_out != nullptr;
+      if (PAY != PAY_NONE && !caller_keys) first.keys_for_fixup = S + plan.off_uf_keys;
+      radix_sort_passes<KeyT, PAY>(L, plan, a, first);
+      done_flag = flags + 1;
+    }
+  }
+  RadixRun all;
+  all.done_flag = done_flag;
+  radix_sort_passes<KeyT, PAY>(L, plan, a, all);
+}
+
+template <typename KeyT, int PAY>
+static void radix_sort_passes(Launcher& L, const Plan& plan, const SortArgs& a, const RadixRun& run)
 {
   const size_t eb    = sizeof(KeyT);
   const char* vin    = reinterpret_cast<const char*>(a.values_in);
@@ -751,6 +829,10 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   // of place the input outlives the sort, they are taken from there at the end, and passes
   // may be skipped as in every other sort.
   Plan pl                  = plan;
+  if (run.upper_first) {
+    pl.n_passes -= run.digit_base;
+    pl.early_last = 0;  // (the pass over the most significant digit writes the result)
+  }
   const bool specials_late = pl.specials && vin != vout;
   if (specials_late && skip_passes_default() && pl.n_passes >= 3) {
     pl.skip_dead_passes = true;
@@ -763,17 +845,6 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
     reinterpret_cast<unsigned long long*>(S + pl.off_special_ctr);
   unsigned long long* special_blk =
     reinterpret_cast<unsigned long long*>(S + pl.off_special_blk);
-
-  // few distinct keys: the four-launch path writes the result, and the kernels below return at once
-  const uint32_t* done_flag = nullptr;
-  if constexpr (sizeof(KeyT) == 4 || sizeof(KeyT) == 8) {
-    const bool outputs_apart = (a.values_out == nullptr || a.values_out != a.values_in) &&
-                               (a.indices_out == nullptr || a.indices_out != a.indices_in);
-    if (pl.low_card && outputs_apart) {
-      bucket_sort_row<KeyT, PAY>(L, pl, a, pl.low_card);
-      done_flag = reinterpret_cast<const uint32_t*>(S + pl.off_bk_flags) + 1;
-    }
-  }
 
   launch_zero(L, S + pl.off_special_ctr, pl.zero_bytes);
 
@@ -798,7 +869,9 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   pp.slabs_per_row   = (uint32_t)pl.slabs_per_row;
   pp.xform           = pl.dt.xform;
   pp.rank_by_add     = rank_by_add_on_current_device();
-  pp.done_flag       = done_flag;
+  pp.done_flag       = run.done_flag;
+  pp.go_flag         = run.go_flag;
+  pp.digit_base      = run.digit_base;
   pp.n_rows          = (uint32_t)pl.rows;
   pp.key_buf[0]      = S + pl.off_keys[0];
   pp.key_buf[1]      = S + pl.off_keys[1];
@@ -813,7 +886,7 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
   else if (alias_keys)
     final_keys = S + pl.off_keys[0];
   else
-    final_keys = write_keys_last ? vout : nullptr;
+    final_keys = write_keys_last ? vout : run.keys_for_fixup;
   if (PAY != PAY_NONE) {
     if (pl.gather_values)
       final_pay = S + pl.off_gather_idx;
@@ -841,7 +914,7 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
     pp.keys_out = dst_keys;
     pp.pay_in   = cur_pay;
     pp.pay_out  = dst_pay;
-    pp.shift    = pass * RADIX_BITS;
+    pp.shift    = (pass + run.digit_base) * RADIX_BITS;
     {
       uint8_t* side = (pl.side_band || pl.side_adaptive) ? reinterpret_cast<uint8_t*>(S + pl.off_digits) : nullptr;
       pp.digits_in  = first ? nullptr : side;  // written by the pass before
@@ -902,6 +975,30 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
 
   if (alias_keys) launch_copy(L, K_COPY, vout, S + pl.off_keys[0], pl.volume * eb);
   if (alias_pay) launch_copy(L, K_COPY, iout, S + pl.off_pay[0], pl.volume * pay_bytes);
+
+  if constexpr (sizeof(KeyT) == 8) {
+    if (run.upper_first) {
+      // the result is in order of the upper digits: runs of equal upper digits by the whole key
+      UpperFirstParams up{};
+      up.volume  = pl.volume;
+      up.row_len = pl.row_len;
+      up.xform    = pl.dt.xform;
+      up.low_bits = RADIX_BITS * run.digit_base;
+      up.flags    = reinterpret_cast<uint32_t*>(S + pl.off_uf_flags);
+      up.elems   = final_keys;
+      up.pos     = PAY != PAY_NONE ? reinterpret_cast<int64_t*>(final_pay) : nullptr;
+      const size_t per = (size_t)UF_FIX_NT * UF_FIX_IPT;
+      const size_t cpr = (pl.row_len + per - 1) / per;
+      L.run(K_UF_FIXUP, [&] {
+        if (PAY != PAY_NONE)
+          hipLaunchKernelGGL((upper_first_fixup_kernel<KeyT, true>), dim3((unsigned)(pl.rows * cpr)), dim3(UF_FIX_NT), 0,
+                             L.stream, up, (uint32_t)cpr);
+        else
+          hipLaunchKernelGGL((upper_first_fixup_kernel<KeyT, false>), dim3((unsigned)(pl.rows * cpr)), dim3(UF_FIX_NT),
+                             0, L.stream, up, (uint32_t)cpr);
+      });
+    }
+  }
 
   if constexpr (is_float_width<KeyT>() && PAY == PAY_NONE) {
     if (specials_late) {
@@ -1138,6 +1235,7 @@ static int partition_layout(int dtype, size_t volume, size_t sort_dim_size, bool
   PlanOptions radix_only;
   radix_only.bucket_path     = 0;
   radix_only.low_cardinality = 0;
+  radix_only.upper_first     = 0;
   int rc = make_plan(dtype, volume, sort_dim_size, want_indices, false, u.pl, radix_only);
   if (rc != MISORT_OK) return rc;
   // 1- and 2-byte values are counted, which beats selecting; their positions are selected
@@ -1518,6 +1616,7 @@ static PlanOptions plan_options(const misort_options* o)
     opt.low_cardinality      = o->low_cardinality;
     opt.bucket_oversample    = o->bucket_oversample;
     opt.counting_sort        = o->counting_sort;
+    opt.upper_first          = o->upper_first;
   }
   return opt;
 }
@@ -1627,6 +1726,10 @@ int misort_describe_plan_opts(int dtype, size_t volume, size_t sort_dim_size, in
   if (pl.low_card) {
     const size_t len = strlen(buf);
     if (len + 32 < buf_bytes) snprintf(buf + len, buf_bytes - len, " low_cardinality_attempt=%d", pl.low_card);
+  }
+  if (pl.upper_first) {
+    const size_t len = strlen(buf);
+    if (len + 32 < buf_bytes) snprintf(buf + len, buf_bytes - len, " upper_first_attempt=%d", pl.upper_first);
   }
   if (pl.skip_dead_passes) {
     const size_t len = strlen(buf);

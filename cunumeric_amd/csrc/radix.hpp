@@ -67,6 +67,8 @@ struct PassParams {
                              // for the row (passes that decide it per row)
   uint32_t n_rows;
   int pass, n_passes;        // which pass this is, of how many
+  int digit_base;            // pass j runs over digit digit_base + j of the key (0 unless the sort is by
+                             // the upper digits only, upperfirst.hpp); shift = 8 * (digit_base + pass)
   // Passes whose digit is the same in every key move nothing and are skipped, decided on the
   // device: the first upsweep ORs all keys and all complemented keys into key_bits_out
   // (KEY_BITS_SLOTS copies of {or lo, or hi, or-of-complement lo, hi}); a bit varies iff it
@@ -105,7 +107,16 @@ struct PassParams {
   // if that path has written the result already, and every kernel of the radix path then
   // returns at once.
   const uint32_t* done_flag;
+  // Non-NULL in the kernels of a sort by the upper digits that is tried first: they run only if
+  // the word is non-zero (the sample said that it pays).
+  const uint32_t* go_flag;
 };
+
+// (every kernel of a pass starts with this)
+__device__ __forceinline__ bool pass_called_off(const PassParams& p)
+{
+  return (p.done_flag && *p.done_flag) || (p.go_flag && *p.go_flag == 0);
+}
 
 // key_bits holds this many copies of its four words (their OR counts)
 constexpr int KEY_BITS_SLOTS = 8;
@@ -148,7 +159,9 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
   // both signs: 0x00 / 0xFF) needs no pass either, since the pass over the most significant
   // digit, which then runs because the sign varies, puts the signs apart; the words say that
   // of the values with their sign extension taken out.
-  const bool by_magnitude = p.xform == XF_SIGNED && p.n_passes <= 8;
+  const int base          = p.digit_base;             // pass j <-> digit base + j
+  const int top_digit     = base + p.n_passes - 1;    // the most significant digit of the key
+  const bool by_magnitude = p.xform == XF_SIGNED && top_digit < 8;
   // bit j: no key varies in digit j (or only with the sign).  Worked out once for all digits:
   // choosing between the words digit by digit where they are used made the compiler keep them
   // in scratch memory.
@@ -156,10 +169,10 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const bool in_lo = ((lo >> (8 * j)) & 0xFFull) == 0, in_hi = ((hi >> (8 * j)) & 0xFFull) == 0;
-    constant_digits |= (uint32_t)((by_magnitude && j < p.n_passes - 1) ? in_hi : in_lo) << j;
+    constant_digits |= (uint32_t)((by_magnitude && j < top_digit) ? in_hi : in_lo) << j;
     constant_digits |= (uint32_t)in_hi << (j + 8);  // digits 8 .. 15 of 16-byte keys
   }
-  auto constant = [&](int j) { return ((constant_digits >> j) & 1u) != 0; };
+  auto constant = [&](int j) { return ((constant_digits >> (j + base)) & 1u) != 0; };  // j: a pass
   // the last pass that runs
   int last = p.n_passes - 1;
   if (p.early_last) {
@@ -172,15 +185,15 @@ __device__ __forceinline__ PassPlan plan_pass(const PassParams& p)
   r.is_last = p.pass == last;
   int nx = p.pass + 1;
   while (nx < last && dead(nx)) ++nx;
-  r.next_shift = nx * RADIX_BITS;
+  r.next_shift = (nx + base) * RADIX_BITS;
   int pv = p.pass - 1;
   while (pv > 0 && dead(pv)) --pv;
   r.prev_live = pv;
   {
     // (a pass that runs over a constant digit is the one over the most significant digit,
     // which the words of the keys themselves describe)
-    const unsigned long long ones = uniform64(p.pass < 8 ? w[0] : w[1]);
-    const int sh = 8 * (p.pass & 7);
+    const unsigned long long ones = uniform64(p.pass + base < 8 ? w[0] : w[1]);
+    const int sh = 8 * ((p.pass + base) & 7);
     if (constant(p.pass) && !(by_magnitude && p.pass < p.n_passes - 1))
       r.const_digit = (int)((ones >> sh) & 0xFFull);
   }
@@ -293,7 +306,7 @@ template <int NT>
 __global__ void __launch_bounds__(NT) upsweep_digits_kernel(PassParams p)
 {
   __shared__ __attribute__((aligned(16))) uint32_t h[RADIX * 32];
-  if (p.done_flag && *p.done_flag) return;
+  if (pass_called_off(p)) return;
   for (int i = threadIdx.x; i < RADIX * 32; i += NT) h[i] = 0;  // (while the plan's words arrive)
   const bool skip = plan_pass(p).skip;
   __syncthreads();
@@ -317,7 +330,7 @@ __global__ void __launch_bounds__(NT) upsweep_kernel(PassParams p)
   constexpr int WORDS  = NW * RADIX * COPIES > RADIX * 32 ? NW * RADIX * COPIES : RADIX * 32;
   __shared__ __attribute__((aligned(16))) uint32_t lhist[WORDS];
   __shared__ unsigned long long wg_bits[FIRST ? NW * 4 : 1];
-  if (p.done_flag && *p.done_flag) return;
+  if (pass_called_off(p)) return;
   const uint32_t row   = blockIdx.x / p.chunks_per_row;
   const uint32_t chunk = blockIdx.x % p.chunks_per_row;
   // (the counters are cleared while the words of the plan arrive)
@@ -622,7 +635,7 @@ __global__ void __launch_bounds__(NT, OCC) downsweep_kernel(PassParams p)
   __shared__ unsigned long long b_pos[SIDE ? RADIX : 1];
   __shared__ uint32_t b_tab[SIDE ? RADIX : 1];
 
-  if (p.done_flag && *p.done_flag) return;
+  if (pass_called_off(p)) return;
   const int tid        = threadIdx.x;
   const int lane       = tid & 63;
   const int wave       = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -112,6 +112,14 @@ def sort_swapped(
         sort_result = output._empty_like_shape(swapped_copy.shape)
         sort(sort_result, swapped_copy, argsort, stable=stable, kth=kth)
         output._rebind(sort_result._swap_with_last(sort_axis))
+    elif swapped_copy.dtype.itemsize == 8 and swapped_copy.size >= (1 << 25) and kth is None:
+        # long sorts of 8-byte keys are quicker out of place: the library then tries the radix
+        # passes over the upper bytes only first, which it cannot do where the result
+        # overwrites the input (the reference sorts the copy in place, cunumeric/sort.py:62-70)
+        sort_result = output._empty_like_shape(swapped_copy.shape)
+        sort(sort_result, swapped_copy, argsort, stable=stable, kth=kth)
+        del swapped_copy
+        output._rebind(sort_result._swap_with_last(sort_axis))
     else:
         sort(swapped_copy, swapped_copy, argsort, stable=stable, kth=kth)
         output._rebind(swapped_copy._swap_with_last(sort_axis))

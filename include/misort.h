@@ -279,6 +279,13 @@ int misort_local_chunked(int dtype, const void* values_in, void* values_out, con
  *                         counters) instead of radix-sorted.  < 0: built in (from 2^24 float16
  *                         and 2^26 integer elements on, where counting is ahead); 0: never;
  *                         > 0: every such row that is too long for the row kernels
+ *   upper_first           long sorts of 8-byte keys (outputs apart from the inputs) run their
+ *                         radix passes over the upper five bytes only, and one read of the
+ *                         result then sorts the short runs of keys that agree in those; a
+ *                         sample of the keys decides whether that is tried, and the eight
+ *                         passes follow on the device if a run was too long to sort that way.
+ *                         < 0: built in (from 2^25 elements on); 0: never; 1: any length;
+ *                         2: tried whatever the sample says (tests of the way back)
  */
 typedef struct misort_options {
   size_t target_chunks;
@@ -289,6 +296,7 @@ typedef struct misort_options {
   int low_cardinality;
   unsigned bucket_oversample;
   int counting_sort;
+  int upper_first;
 } misort_options;
 size_t misort_scratch_bytes_opts(int dtype, size_t volume, size_t sort_dim_size, int argsort,
                                  int has_indices_in, const misort_options* options);
