@@ -112,7 +112,9 @@ def test_float_zeros_and_nans_keep_their_bits(abi):
     a[rng.integers(0, n, 50)] = -np.inf
     for mode in (1, 2):
         check(abi, a, n, mode)
-    c = (a[: n // 2] + 1j * a[n // 2: 2 * (n // 2)]).astype(np.complex64)
+    c = np.empty(n // 2, dtype=np.complex64)
+    c.real = a[: n // 2]
+    c.imag = a[n // 2: 2 * (n // 2)]
     for mode in (1, 2):
         check(abi, c, c.size, mode)
 
@@ -139,3 +141,21 @@ def test_built_in_choice_starts_at_two_to_the_25(abi):
     assert "upper_first_attempt" not in abi.describe_plan(np.float32, 1 << 26, 1 << 26, True)
     assert "upper_first_attempt" not in abi.describe_plan(np.complex128, 1 << 25, 1 << 25, True)
     assert "upper_first_attempt" not in abi.describe_plan(np.int64, 1 << 26, 1 << 26, True, options=Options(upper_first=0))
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.float64, np.complex64], ids=lambda d: np.dtype(d).name)
+def test_two_to_the_25_elements_with_the_built_in_choice(abi, dtype):
+    """The size from which the attempt is made by itself: uniform keys (a handful of pairs agree
+    in their upper bits), against numpy's stable sort."""
+    rng = np.random.default_rng(95)
+    n = 1 << 25
+    if np.dtype(dtype).kind == "i":
+        a = rng.integers(-2**63, 2**63 - 1, n, dtype=np.int64)
+    elif np.dtype(dtype).kind == "f":
+        a = rng.standard_normal(n)
+    else:
+        a = (rng.standard_normal(n, dtype=np.float32) + 1j * rng.standard_normal(n, dtype=np.float32)).astype(np.complex64)
+    assert "upper_first_attempt=1" in abi.describe_plan(dtype, n, n, True)
+    print(f"upper first 2^25 dtype={np.dtype(dtype).name}", flush=True)
+    assert np.array_equal(abi.local_sort(a, n, argsort=True), np.argsort(a, kind="stable"))
+    assert bits_equal(abi.local_sort(a, n, argsort=False), np.sort(a, kind="stable"))
