@@ -5,7 +5,7 @@
 
 One "step" is one call of the hot path (misort_local through the C ABI) over the whole
 batch: float32 keys in HBM -> int64 stable-argsort indices in HBM.  Prints ONE JSON line.
---workload selects one of the other benchmark inputs (c1, c3, c3t, c4, c5a, c5b) for the
+--workload selects one of the other benchmark inputs (c1, c3, c3t, c4, c5a, c5b, i64, f64) for the
 same line format; the default, c2, is the headline.  Every run of these workloads ends with
 plain 1 GiB device copies: their rate is reported beside the roofline, and they give
 hardware-counter runs a kernel of known traffic to scale by (--calib-copy is accepted for
@@ -71,6 +71,16 @@ def make_c4(n: int = 1 << 28, seed: int = 4) -> np.ndarray:
     v = rng.integers(-(2**63), 2**63, 16, dtype=np.int64)
     w = np.arange(1, 17, dtype=np.float64) ** -1.2
     return v[rng.choice(16, n, p=w / w.sum())]
+
+
+def make_uniform_int64(n: int = 1 << 28, seed: int = 9) -> np.ndarray:
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return rng.integers(-(2**63), 2**63 - 1, n, dtype=np.int64, endpoint=True)
+
+
+def make_normal_float64(n: int = 1 << 28, seed: int = 10) -> np.ndarray:
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return rng.standard_normal(n)
 
 
 def make_small_int64(n: int = 1 << 28, seed: int = 8) -> np.ndarray:
@@ -204,6 +214,10 @@ WORKLOADS = {
     "c5b": ("C5b: 1-D float16 uniform(-1,1), sort (keys only)", make_c5b, 30, False, 0),
     "i64small": ("1-D int64 below 50000, stable argsort (six of the eight radix passes see one "
                  "digit value and are skipped)", make_small_int64, 28, True, 0),
+    "i64": ("1-D int64 full range, stable argsort (the radix passes run over the upper five key "
+            "bytes, one read of the result sorts the runs of equal upper bytes)", make_uniform_int64, 28, True, 0),
+    "f64": ("1-D float64 N(0,1), stable argsort (radix passes over the upper six key bytes first)",
+            make_normal_float64, 28, True, 0),
 }
 
 # HBM bytes per launch of the downsweep kernel on the headline workload (N = 2^28), from
@@ -889,7 +903,9 @@ def main() -> int:
                 ran = np.zeros_like(per_launch, dtype=bool)
             elif name == "upsweep":
                 ran = per_launch >= 0.05 * per_launch.max()
-            elif name in ("downsweep_middle", "downsweep_last"):
+            elif name.startswith("downsweep_"):
+                # (with an attempt by the upper bytes first, plan upper_first_attempt, the launches
+                # of the eight-pass sort follow and return at once, its first pass included)
                 ran = per_launch >= 0.05 * longest_scatter
             else:
                 ran = np.ones_like(per_launch, dtype=bool)
@@ -916,6 +932,8 @@ def main() -> int:
         for name, kk in kernels.items():
             if name.startswith("downsweep_"):
                 b = algorithmic_bytes_per_key(k_bytes, v_bytes, name)
+            elif name == "upper_first_fixup":
+                b = k_bytes  # one read of the result's keys (the runs it sorts are a few per mille)
             elif name.startswith("rowsort_"):
                 b, dominant = 2 * k_bytes + v_bytes, name
             elif name in ("count16_hist", "count16_fill"):

@@ -156,10 +156,20 @@ __global__ void __launch_bounds__(UF_FIX_NT) upper_first_fixup_kernel(UpperFirst
   const int lb = p.low_bits;
   auto upper   = [&](KeyT e) { return key(e) >> lb; };
   const uint64_t c0 = (uint64_t)chunk * (NT * IPT);
+  // every thread's elements and their right neighbours, all loads in flight at once (a run that
+  // another thread is sorting meanwhile may be seen half sorted: see below)
+  KeyT ea[IPT], eb[IPT];
+#pragma unroll
+  for (int j = 0; j < IPT; ++j) {
+    const uint64_t i = c0 + (uint64_t)j * NT + threadIdx.x;
+    ea[j]            = el[i < n ? i : n - 1];
+    eb[j]            = el[i + 1 < n ? i + 1 : n - 1];
+  }
+#pragma unroll
   for (int j = 0; j < IPT; ++j) {
     const uint64_t i = c0 + (uint64_t)j * NT + threadIdx.x;
     if (i + 1 >= n) continue;  // (the last element of a row has no right neighbour; it may end a run)
-    const KeyT a = key(el[i]), b = key(el[i + 1]);
+    const KeyT a = key(ea[j]), b = key(eb[j]);
     if ((a >> lb) != (b >> lb)) continue;
     const KeyT up = a >> lb;
     // The upper bits of a place never change (runs are permuted inside themselves only), so
