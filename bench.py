@@ -805,6 +805,26 @@ def main() -> int:
     ms_per_step = elapsed / args.steps * 1e3
     gkeys = n / (elapsed / args.steps) / 1e9
 
+    # Where the sort ran by the upper key bytes first (plan upper_first_attempt): the same call
+    # with all eight passes, for comparison (misort_options.upper_first = 0)
+    eight_pass_ms = None
+    if not host_api and "upper_first_attempt" in plan:
+        from cunumeric_amd._lib import Options
+
+        o8 = Options(upper_first=0)
+        for _ in range(max(args.warmup, 1)):
+            _lib.check(lib.misort_local_opts(code, d_in.data_ptr(), vo, None, io, n, row_len, 1, 0,
+                                             scratch.data_ptr(), need, stream, ctypes.byref(o8)))
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            _lib.check(lib.misort_local_opts(code, d_in.data_ptr(), vo, None, io, n, row_len, 1, 0,
+                                             scratch.data_ptr(), need, stream, ctypes.byref(o8)))
+        torch.cuda.synchronize()
+        eight_pass_ms = (time.perf_counter() - t1) / args.steps * 1e3
+        step()  # (the output checked below is the default call's)
+        torch.cuda.synchronize()
+
     # One call at a time: HIP events on the launch stream (torch's current stream is the one
     # handed to the library) from before the first launch to after the last kernel of the
     # call, the device idle before each call; median over the calls.
@@ -1061,6 +1081,7 @@ def main() -> int:
         "ms_per_step": ms_per_step,
         # one call timed alone with HIP events (median of n), and its throughput
         "call_ms_median": call_ms,
+        **({"ms_per_step_all_eight_passes": eight_pass_ms} if eight_pass_ms is not None else {}),
         "call_ms_n": n_ev,
         "value_per_call": n / (call_ms * 1e-3) / 1e9,
         "device_copy_GBs": copy_gbs,
