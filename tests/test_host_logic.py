@@ -69,6 +69,51 @@ def test_describe_plan(lib):
     assert "passes=2" in _lib.describe_plan(9, 1 << 22, 1 << 21, False)  # two rows: radix
 
 
+def test_plans_of_the_paths_beside_the_radix_passes(lib):
+    """Where the four-launch path, the counting sort and the two attempts of long radix sorts
+    are planned (type codes of include/misort.h: 1 int8, 2 int16, 3 int32, 4 int64, 9 float16,
+    10 float32, 11 float64, 12 complex64, 13 complex128)."""
+    from cunumeric_amd._lib import Options
+
+    plan = _lib.describe_plan
+    bucket = lambda code, vol, row, arg, **kw: "strategy=bucket" in plan(code, vol, row, arg, **kw)
+    # medium rows: four launches, up to where the radix passes catch up
+    assert bucket(3, 1 << 20, 1 << 20, False) and bucket(3, 1 << 21, 1 << 21, True)
+    assert not bucket(3, (1 << 21) + 1, (1 << 21) + 1, False)
+    assert bucket(3, 3 << 19, 3 << 16, True) and not bucket(3, 1 << 21, 1 << 18, True)   # several rows
+    assert bucket(11, 1 << 21, 1 << 21, True) and bucket(4, 1 << 22, 1 << 19, False)
+    assert not bucket(4, 1 << 23, 1 << 19, False)
+    assert bucket(2, 1 << 19, 1 << 19, False) and not bucket(2, 1 << 20, 1 << 20, False)
+    assert bucket(9, 1 << 20, 1 << 20, False) and not bucket(9, 1 << 19, 1 << 19, True)
+    assert not bucket(1, 1 << 16, 1 << 16, True) and not bucket(13, 1 << 16, 1 << 16, True)
+    assert bucket(1, 1 << 16, 1 << 16, True, options=Options(bucket_path=1))
+    assert not bucket(3, 1 << 18, 1 << 18, False, options=Options(bucket_path=0))
+    assert "bin_cap=16384" in plan(4, 1 << 20, 1 << 20, True)
+    # counting sort of 2-byte values
+    assert "strategy=count16" in plan(9, 1 << 24, 1 << 24, False)
+    assert "strategy=count16" not in plan(2, 1 << 24, 1 << 24, False)
+    assert "strategy=count16" in plan(2, 1 << 26, 1 << 26, False)
+    assert "strategy=count16" in plan(2, 1 << 20, 1 << 20, False, options=Options(counting_sort=1))
+    assert "strategy=count16" not in plan(2, 1 << 26, 1 << 26, False, options=Options(counting_sort=0))
+    # long radix sorts: few distinct keys, and 8-byte keys by their upper bytes first
+    assert "low_cardinality_attempt=1" in plan(10, 1 << 27, 1 << 27, True)
+    assert "low_cardinality_attempt" not in plan(10, 1 << 26, 1 << 26, True)
+    assert "upper_first_attempt=1" in plan(11, 1 << 25, 1 << 25, False)
+    assert "upper_first_attempt=1" in plan(12, 1 << 26, 1 << 20, True)
+    assert "upper_first_attempt" not in plan(11, (1 << 25) - 1, (1 << 25) - 1, False)
+    assert "upper_first_attempt" not in plan(10, 1 << 28, 1 << 28, True)
+    assert "upper_first_attempt" not in plan(13, 1 << 26, 1 << 26, True)
+    assert "upper_first_attempt=2" in plan(4, 1 << 22, 1 << 22, True, options=Options(bucket_path=0, upper_first=2))
+    assert "upper_first_attempt" not in plan(4, 1 << 26, 1 << 26, True, options=Options(upper_first=0))
+    # the attempt's fix-up needs the keys of an argsort's result: 8 bytes per element more scratch
+    n = 1 << 26
+    with_keys = lib.misort_scratch_bytes(4, n, n, 1, 0)
+    import ctypes
+    o = Options(upper_first=0)
+    without = lib.misort_scratch_bytes_opts(4, n, n, 1, 0, ctypes.byref(o))
+    assert 8 * n <= with_keys - without <= 8 * n + 4096
+
+
 def test_argument_errors_need_no_gpu(lib):
     def call(dtype, vin, vout, iin, iout, volume, row, scratch, sbytes):
         return lib.misort_local(dtype, vin, vout, iin, iout, volume, row, 1, 0, scratch, sbytes, None)
