@@ -794,7 +794,7 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
       up.volume      = plan.volume;
       up.row_len     = plan.row_len;
       up.xform       = plan.dt.xform;
-      up.low_bits    = RADIX_BITS * upper_first_digit0(plan.dt.xform);
+      up.low_bits    = RADIX_BITS * upper_first_digit0(plan.dt.xform, plan.row_len);
       up.mode        = plan.upper_first;
       up.rank_by_add = rank_by_add_on_current_device();
       up.flags       = flags;
@@ -803,7 +803,7 @@ static void radix_sort_rows(Launcher& L, const Plan& plan, const SortArgs& a)
         hipLaunchKernelGGL((upper_first_plan_kernel<KeyT>), dim3(1), dim3(UF_PLAN_NT), 0, L.stream, up);
       });
       RadixRun first;
-      first.digit_base  = upper_first_digit0(plan.dt.xform);
+      first.digit_base  = upper_first_digit0(plan.dt.xform, plan.row_len);
       first.go_flag     = flags;
       first.upper_first = true;
       const bool caller_keys = !plan.argsort || a.values_out != nullptr;
@@ -1729,7 +1729,9 @@ int misort_describe_plan_opts(int dtype, size_t volume, size_t sort_dim_size, in
   }
   if (pl.upper_first) {
     const size_t len = strlen(buf);
-    if (len + 32 < buf_bytes) snprintf(buf + len, buf_bytes - len, " upper_first_attempt=%d", pl.upper_first);
+    if (len + 48 < buf_bytes)
+      snprintf(buf + len, buf_bytes - len, " upper_first_attempt=%d upper_digits=%d", pl.upper_first,
+               8 - upper_first_digit0(pl.dt.xform, pl.row_len));
   }
   if (pl.skip_dead_passes) {
     const size_t len = strlen(buf);

@@ -1,13 +1,13 @@
-// Long sorts of 8-byte keys, tried by the upper 40 or 48 bits first.
+// Long sorts of 8-byte keys, tried by the upper 32 to 48 bits first.
 //
 // Eight radix passes move every key eight times; the lower bytes only matter for keys that
 // agree in the upper ones, and among 2^28 keys drawn from 64-bit integers a few thousand pairs
-// agree in their upper 40 bits.  So the radix passes run over digits 3 .. 7 only (five passes
-// instead of eight; PassParams::digit_base), which leaves the keys in order up to short runs
-// of equal upper bits, and one more read of the result puts those runs right.  Float keys
-// spend 12 of their upper bits on sign and exponent, which a few values share between all
-// keys (2^27 uniform doubles: a quarter of the keys in runs of equal upper 40 bits; complex64:
-// the real parts alone collide), so they keep their upper 48 bits (six passes):
+// agree in their upper 40 bits.  So the radix passes run over the upper four to
+// six digits only (PassParams::digit_base; upper_first_digit0 below picks how many from the
+// row length and the kind of key), which leaves the keys in order up to short runs of equal
+// upper bits, and one more read of the result puts those runs right.  Float keys spend 12 of
+// their upper bits on sign and exponent, which a few values share between all keys (2^27
+// uniform doubles: a quarter of the keys in runs of equal upper 40 bits), so they keep more:
 //
 //   upper_first_plan_kernel   one workgroup sorts a sample of 8192 keys and lets the attempt go
 //                             on only if no two sample keys agree in the upper bits while
@@ -35,8 +35,24 @@
 
 namespace misort {
 
-// digits left to the fix-up: three of integer keys, two of float and complex keys
-__host__ __device__ constexpr int upper_first_digit0(int xform) { return xform == XF_FLOAT || xform == XF_COMPLEX ? 2 : 3; }
+// Digits left to the fix-up.  The passes keep the fewest upper bytes for which a row's keys,
+// spread evenly, would have an expected run length of 1/64 or less: log2(row length) + 6 bits,
+// plus what the key's upper bits do not spend on telling values apart (sign and exponent of a
+// double: 12; the signs and exponents of both parts of a complex64 and the mantissa bits that
+// its real part lacks: 15).  Sorting a run costs its thread a handful of dependent reads and
+// writes while its wavefront waits: with one key in sixteen in a run (2^28 int64 by their
+// upper 32 bits) the fix-up took 3.9 ms instead of 0.55, more than the pass it saved.
+// 2^25 int64: 32 bits (four passes); 2^28 int64: 40; rows of 2^20 doubles: 40; 2^28: 48.
+static inline int upper_first_digit0(int xform, uint64_t row_len)
+{
+  const int spent = xform == XF_FLOAT ? 12 : xform == XF_COMPLEX ? 15 : 0;
+  int need        = 6 + spent;
+  while (need < 64 && (row_len >> (need - 6 - spent)) > 1) ++need;
+  int bytes = (need + 7) / 8;
+  if (bytes < 4) bytes = 4;
+  if (bytes > 6) bytes = 6;
+  return 8 - bytes;
+}
 constexpr int UF_RUN_LIMIT = 16;  // longest run the fix-up sorts
 constexpr int UF_PLAN_NT   = 1024;
 constexpr int UF_PLAN_IPT  = 8;   // 8192 sample keys
