@@ -36,18 +36,19 @@
 namespace misort {
 
 // Digits left to the fix-up.  The passes keep the fewest upper bytes for which a row's keys,
-// spread evenly, would have an expected run length of 1/64 or less: log2(row length) + 6 bits,
+// spread evenly, would have an expected run length of 1/32 or less: log2(row length) + 5 bits,
 // plus what the key's upper bits do not spend on telling values apart (sign and exponent of a
 // double: 12; the signs and exponents of both parts of a complex64 and the mantissa bits that
-// its real part lacks: 15).  Sorting a run costs its thread a handful of dependent reads and
-// writes while its wavefront waits: with one key in sixteen in a run (2^28 int64 by their
-// upper 32 bits) the fix-up took 3.9 ms instead of 0.55, more than the pass it saved.
-// 2^25 int64: 32 bits (four passes); 2^28 int64: 40; rows of 2^20 doubles: 40; 2^28: 48.
+// its real part lacks: 15).  Runs of two are exchanged in passing, but a longer run costs its
+// thread a dozen dependent reads and writes while its wavefront waits: with one key in sixteen
+// in a run (2^28 int64 by their upper 32 bits) the fix-up took 2.5 ms instead of 0.55, as much
+// as the pass it saved; at one in thirty-two (2^27) the sort is 8 % quicker with four passes.
+// 2^27 int64: 32 bits (four passes); 2^28 int64: 40; rows of 2^20 doubles: 40; 2^28: 48.
 static inline int upper_first_digit0(int xform, uint64_t row_len)
 {
   const int spent = xform == XF_FLOAT ? 12 : xform == XF_COMPLEX ? 15 : 0;
-  int need        = 6 + spent;
-  while (need < 64 && (row_len >> (need - 6 - spent)) > 1) ++need;
+  int need        = 5 + spent;
+  while (need < 64 && (row_len >> (need - 5 - spent)) > 1) ++need;
   int bytes = (need + 7) / 8;
   if (bytes < 4) bytes = 4;
   if (bytes > 6) bytes = 6;
@@ -181,13 +182,26 @@ __global__ void __launch_bounds__(UF_FIX_NT) upper_first_fixup_kernel(UpperFirst
     ea[j]            = el[i < n ? i : n - 1];
     eb[j]            = el[i + 1 < n ? i + 1 : n - 1];
   }
+  const int lane    = threadIdx.x & 63;
+  uint32_t exchange = 0;  // bit j: elements i and i + 1 of slot j are a run of two in the wrong order
 #pragma unroll
   for (int j = 0; j < IPT; ++j) {
     const uint64_t i = c0 + (uint64_t)j * NT + threadIdx.x;
-    if (i + 1 >= n) continue;  // (the last element of a row has no right neighbour; it may end a run)
     const KeyT a = key(ea[j]), b = key(eb[j]);
+    // the elements before and after the pair are the neighbouring lanes' (every lane takes
+    // part in the exchange; the wavefront's first and last lane read theirs if they need them)
+    KeyT before = __shfl_up(ea[j], 1, 64), after = __shfl_down(eb[j], 1, 64);
+    if (i + 1 >= n) continue;  // (the last element of a row has no right neighbour; it may end a run)
     if ((a >> lb) != (b >> lb)) continue;
     const KeyT up = a >> lb;
+    if (lane == 0 && i > 0) before = el[i - 1];
+    if (lane == 63 && i + 2 < n) after = el[i + 2];
+    const bool first = i == 0 || upper(before) != up;
+    if (first && (i + 2 >= n || upper(after) != up)) {
+      // a run of two, nearly all there are: in order, or exchanged below
+      if (a > b) exchange |= 1u << j;
+      continue;
+    }
     // The upper bits of a place never change (runs are permuted inside themselves only), so
     // the extent of a run is safe to read while another thread sorts it; the whole keys of a
     // short run may be read half way through its sorting, which only matters for long runs,
@@ -202,7 +216,7 @@ __global__ void __launch_bounds__(UF_FIX_NT) upper_first_fixup_kernel(UpperFirst
         continue;
       }
     }
-    if (i > 0 && upper(el[i - 1]) == up) continue;  // not the first of its run
+    if (!first) continue;  // not the first of its run
     uint64_t e = i + 2;
     while (e < n && e - i <= (uint64_t)UF_RUN_LIMIT && upper(el[e]) == up) ++e;
     if (e - i > (uint64_t)UF_RUN_LIMIT) continue;  // (in order already, or called off above)
@@ -223,6 +237,34 @@ __global__ void __launch_bounds__(UF_FIX_NT) upper_first_fixup_kernel(UpperFirst
       if (y != x) {
         el[y] = ex;
         if constexpr (HAS_POS) pos[y] = px;
+      }
+    }
+  }
+  // the runs of two that are in the wrong order: nobody else touches them, and the values read
+  // at the start are theirs still.  All payload reads of a thread in flight together (one after
+  // the other, each inside its slot's branch, they were most of the kernel's time).
+  if (exchange) {
+    int64_t p0[IPT], p1[IPT];
+    if constexpr (HAS_POS) {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) {
+        const uint64_t i = c0 + (uint64_t)j * NT + threadIdx.x;
+        if ((exchange >> j) & 1u) {
+          p0[j] = pos[i];
+          p1[j] = pos[i + 1];
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < IPT; ++j) {
+      const uint64_t i = c0 + (uint64_t)j * NT + threadIdx.x;
+      if ((exchange >> j) & 1u) {
+        el[i]     = eb[j];
+        el[i + 1] = ea[j];
+        if constexpr (HAS_POS) {
+          pos[i]     = p1[j];
+          pos[i + 1] = p0[j];
+        }
       }
     }
   }
