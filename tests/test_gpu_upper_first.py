@@ -159,3 +159,23 @@ def test_two_to_the_25_elements_with_the_built_in_choice(abi, dtype):
     print(f"upper first 2^25 dtype={np.dtype(dtype).name}", flush=True)
     assert np.array_equal(abi.local_sort(a, n, argsort=True), np.argsort(a, kind="stable"))
     assert bits_equal(abi.local_sort(a, n, argsort=False), np.sort(a, kind="stable"))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_run_structures(abi, seed):
+    """Random lengths, rows, run-length distributions (means from 1 to 12: some runs beyond what
+    the fix-up sorts, so both outcomes of the attempt occur), ties inside runs, every 8-byte type."""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = TYPES[seed % len(TYPES)]
+    rows = int(rng.integers(1, 4))
+    row_len = int(rng.integers(16385, 150000))
+    n = rows * row_len
+    mean = float(rng.choice([1.0, 1.5, 3.0, 6.0, 12.0]))
+    lengths = rng.geometric(1.0 / mean, n)
+    upper = np.repeat(rng.permutation(lengths.size), lengths)[:n] * int(rng.integers(1, 5000))
+    low = rng.integers(0, 1 << int(rng.integers(1, 33)), n)   # (few low bits: ties inside the runs)
+    a = from_keys(dtype, upper[rng.permutation(n)], low)
+    print(f"upper first random seed={seed} dtype={np.dtype(dtype).name} rows={rows} row_len={row_len} mean run={mean}",
+          flush=True)
+    check(abi, a, row_len, 2)
+    check(abi, a, row_len, 1)
