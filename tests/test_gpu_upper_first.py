@@ -50,6 +50,12 @@ def inputs(dtype, n, rng):
     out["long runs"] = from_keys(dtype, rng.integers(0, 500, n) * 100000007, low)
     out["heavy ties"] = out["random"][rng.integers(0, 100, n)]
     out["ties and runs"] = from_keys(dtype, rng.integers(0, n // 4, n) * 1000003, rng.integers(0, 3, n) << 20)
+    # small values of both signs: every upper byte of an integer only repeats the sign, so the
+    # passes over them are skipped or run over two values, and everything is left to the way back
+    small = rng.integers(-1000, 1000, n)
+    out["small, both signs"] = (small + 1j * rng.integers(-3, 3, n)).astype(dtype) if np.dtype(dtype).kind == "c" \
+        else small.astype(dtype) if np.dtype(dtype) != np.uint64 else (small + 1000).astype(dtype)
+    out["wide and small mixed"] = np.where(rng.integers(0, 2, n) == 0, out["small, both signs"], out["random"])
     return out
 
 
