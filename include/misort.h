@@ -25,8 +25,8 @@ extern "C" {
 
 /* Element type codes, in the order of cuNumeric's SUPPORTED_DTYPES table (reference:
  * cunumeric/utils.py:29-44).  They are this library's own numbers: a binding maps its
- * framework's type enumeration to them by name (INTEGRATION.md shows the switch), never by
- * casting one enumeration to the other. */
+ * framework's type enumeration to them by name (a switch over the framework's enumerators
+ * that returns MISORT_<NAME>), never by casting one enumeration to the other. */
 typedef enum misort_dtype {
   MISORT_BOOL       = 0,
   MISORT_INT8       = 1,
