@@ -10,17 +10,18 @@ import itertools
 import pytest
 
 
-def plan(varying_bytes, pass_no, n_passes, early_last=0):
+def plan(varying_bytes, pass_no, n_passes, early_last=0, base=0):
     """(skip, parity, next_live, prev_live, is_last) as plan_pass computes them; early_last: the
-    highest pass that may write the result in place of the top pass (0: none)."""
+    highest pass that may write the result in place of the top pass (0: none); base: pass j runs
+    over byte base + j of the key (PassParams::digit_base: sorts by the upper bytes only)."""
     last = n_passes - 1
     if early_last:
-        while last > 0 and last not in varying_bytes:
+        while last > 0 and last + base not in varying_bytes:
             last -= 1
         if last == 0 or last > early_last:
             last = n_passes - 1
     def dead(j):
-        return j > last or (0 < j < last and j not in varying_bytes)
+        return j > last or (0 < j < last and j + base not in varying_bytes)
     parity = sum(dead(j) for j in range(1, pass_no)) & 1
     nxt = pass_no + 1
     while nxt < last and dead(nxt):
@@ -82,3 +83,33 @@ def test_every_set_of_dead_passes(n_passes, early):
                 assert nxt > k and nxt in runs
             last_live = k
         assert holder == "output"
+
+
+@pytest.mark.parametrize("base", [2, 3, 4])
+def test_sorts_by_the_upper_bytes_only(base):
+    """Passes over bytes base .. 7 of an 8-byte key (the attempt of upperfirst.hpp): what varies
+    in the bytes below base plays no part, pass 0 (byte `base`) always runs, the pass over byte 7
+    writes the result, and the buffers alternate over the live passes as in a sort of all bytes."""
+    n_passes = 8 - base
+    upper = list(range(base + 1, 8))
+    for k in range(len(upper) + 1):
+        for constant in itertools.combinations(upper, k):
+            for low in (set(), set(range(base))):   # the lower bytes constant, or all varying
+                varying = (set(range(base, 8)) - set(constant)) | low
+                runs = {0, n_passes - 1} | {j for j in range(1, n_passes - 1) if j + base in varying}
+                holder, last_live = "input", None
+                for j in range(n_passes):
+                    skip, parity, nxt, prv, is_last = plan(varying, j, n_passes, 0, base)
+                    assert skip == (j not in runs), (base, constant, j)
+                    assert is_last == (j == n_passes - 1)
+                    if skip:
+                        continue
+                    if j:
+                        assert prv == last_live and holder == input_buffer(j, parity)
+                    if is_last:
+                        holder = "output"
+                    else:
+                        holder = input_buffer(j, parity) ^ 1 if j else 0
+                        assert nxt in runs and nxt > j   # the side-band is for byte base + nxt
+                    last_live = j
+                assert holder == "output"
